@@ -1,0 +1,60 @@
+"""Build libgact_hip.so (the C-ABI library of HIP kernels) for gfx950 with hipcc.
+
+    python gact-icml_amd/build.py            # build if the sources are newer than the library
+    python gact-icml_amd/build.py --force
+
+hipcc cross-compiles for gfx950 without a GPU present.  The library lands inside the Python
+package (gact/lib/) so that it travels with the source tree.
+"""
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+SRC = os.path.join(HERE, "csrc", "gact_hip.hip")
+HDR = os.path.join(ROOT, "include", "gact_hip.h")
+OUT_DIR = os.path.join(HERE, "gact", "lib")
+OUT = os.path.join(OUT_DIR, "libgact_hip.so")
+
+HIPCC_FLAGS = [
+    "-O3",
+    "--offload-arch=gfx950",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    # every floating-point operation in the kernels is meant literally (the one FMA is spelled out)
+    "-ffp-contract=off",
+    # keep the compiler from forming packed-FP32 instructions
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def hipcc():
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (set HIPCC)")
+
+
+def up_to_date():
+    if not os.path.exists(OUT):
+        return False
+    t = os.path.getmtime(OUT)
+    return all(os.path.getmtime(p) <= t for p in (SRC, HDR, os.path.abspath(__file__)))
+
+
+def build(force=False, extra=()):
+    if not force and up_to_date():
+        return OUT
+    os.makedirs(OUT_DIR, exist_ok=True)
+    cmd = [hipcc()] + HIPCC_FLAGS + list(extra) + ["-I", os.path.join(ROOT, "include"), "-o", OUT, SRC]
+    subprocess.run(cmd, check=True)
+    return OUT
+
+
+if __name__ == "__main__":
+    print(build(force="--force" in sys.argv))

@@ -1,0 +1,1079 @@
+// GACT saved-activation compression for MI355X (gfx950): per-group min/max, scale, stochastic
+// rounding, bit packing, and the inverse, as hand-written HIP kernels behind a C ABI.
+//
+// Work decomposition (all kernels): a DPP row of 16 lanes owns 8 consecutive groups of 256 elements.
+// Inside a group lane i of the row owns two runs of 8 consecutive columns, 128k + 8i .. +7 (k = 0,1),
+// so every load instruction of a row covers 256 contiguous bytes, per-group reductions are four
+// row_ror DPP steps that never leave the row, and - because the reference packs the SAME column of
+// 8/bits consecutive groups into one byte - the lane that owns a column owns every code of that byte:
+// packing needs no cross-lane traffic at all.  A wave is 4 rows, a workgroup 1 or 4 waves.
+//
+// Floating-point contract: this file is compiled with -ffp-contract=off, so every operation below is
+// the IEEE operation it spells; the one fused multiply-add of the path is written __builtin_fmaf.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <queue>
+#include <utility>
+#include <vector>
+
+#include "gact_hip.h"
+
+typedef _Float16 f16;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+#define GROUP 256
+#define ROW_GROUPS 8 /* groups owned by one 16-lane row */
+
+// ------------------------------------------------------------------------------------------------
+// DPP row reductions (16 lanes).  Rotating by 8, 4, 2, 1 leaves the row-wide result in every lane.
+// ------------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  int x = __builtin_bit_cast(int, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(x, x, CTRL, 0xf, 0xf, false));
+}
+#define DPP_ROW_ROR(n) (0x120 + (n))
+
+__device__ __forceinline__ float row_all_min(float v) {
+  v = __builtin_fminf(v, dpp_f32<DPP_ROW_ROR(8)>(v));
+  v = __builtin_fminf(v, dpp_f32<DPP_ROW_ROR(4)>(v));
+  v = __builtin_fminf(v, dpp_f32<DPP_ROW_ROR(2)>(v));
+  v = __builtin_fminf(v, dpp_f32<DPP_ROW_ROR(1)>(v));
+  return v;
+}
+__device__ __forceinline__ float row_all_max(float v) {
+  v = __builtin_fmaxf(v, dpp_f32<DPP_ROW_ROR(8)>(v));
+  v = __builtin_fmaxf(v, dpp_f32<DPP_ROW_ROR(4)>(v));
+  v = __builtin_fmaxf(v, dpp_f32<DPP_ROW_ROR(2)>(v));
+  v = __builtin_fmaxf(v, dpp_f32<DPP_ROW_ROR(1)>(v));
+  return v;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Philox4x32-10.  The key schedule only depends on the seed, so it stays on the scalar unit.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                              uint32_t k1, uint32_t (&out)[4]) {
+#pragma unroll
+  for (int r = 0; r < 10; r++) {
+    uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c1 = (uint32_t)p1;
+    c3 = (uint32_t)p0;
+    c0 = n0;
+    c2 = n2;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+// cuRAND's uniform map: float(x) * 2^-32 + 2^-33, in (0, 1].  The product is exact, so the fused form
+// rounds once exactly like the separate multiply and add.
+__device__ __forceinline__ float curand_uniform_map(uint32_t x) {
+  return __builtin_fmaf((float)x, 0x1p-32f, 0x1p-33f);
+}
+// 16-bit noise of the fast stream: (h + 0.5) * 2^-16, exact in float.
+__device__ __forceinline__ float fast_uniform_map(uint32_t h) {
+  return __builtin_fmaf((float)h, 0x1p-16f, 0x1p-17f);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Per-type pieces.
+// ------------------------------------------------------------------------------------------------
+template <typename T> struct Elem;
+
+template <> struct Elem<float> {
+  static constexpr int kDtype = GACT_F32;
+  __device__ static __forceinline__ void load8(const float* p, float (&v)[8]) {
+    f32x4 a = *reinterpret_cast<const f32x4*>(p);
+    f32x4 b = *reinterpret_cast<const f32x4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  __device__ static __forceinline__ void store8(float* p, const float (&v)[8]) {
+    f32x4 a = {v[0], v[1], v[2], v[3]};
+    f32x4 b = {v[4], v[5], v[6], v[7]};
+    *reinterpret_cast<f32x4*>(p) = a;
+    *reinterpret_cast<f32x4*>(p + 4) = b;
+  }
+  __device__ static __forceinline__ float to_float(float v) { return v; }
+  __device__ static __forceinline__ float from_float(float v) { return v; }
+  __device__ static __forceinline__ float init_lo() { return 1e30f; }
+  __device__ static __forceinline__ float init_hi() { return -1e30f; }
+  // scale = float( double(float(qmax)) / (double(max - min) + 2e-6) )
+  __device__ static __forceinline__ float make_scale(float lo, float hi, int qmax) {
+    float range = hi - lo;
+    return (float)((double)(float)qmax / ((double)range + 2e-6));
+  }
+  // code = rint(max(fma(x - mn, s, u) - 0.5, 0))
+  __device__ static __forceinline__ int code(float x, float mn, float s, float u) {
+    float t = x - mn;
+    float y = __builtin_fmaf(t, s, u);
+    float z = __builtin_fmaxf(y - 0.5f, 0.0f);
+    return (int)__builtin_rintf(z);
+  }
+  __device__ static __forceinline__ float decode(int c, float s, float mn) {
+    float q = (float)c / s;
+    return q + mn;
+  }
+};
+
+template <> struct Elem<f16> {
+  static constexpr int kDtype = GACT_F16;
+  __device__ static __forceinline__ void load8(const f16* p, f16 (&v)[8]) {
+    f16x8 a = *reinterpret_cast<const f16x8*>(p);
+#pragma unroll
+    for (int e = 0; e < 8; e++) v[e] = a[e];
+  }
+  __device__ static __forceinline__ void store8(f16* p, const f16 (&v)[8]) {
+    f16x8 a;
+#pragma unroll
+    for (int e = 0; e < 8; e++) a[e] = v[e];
+    *reinterpret_cast<f16x8*>(p) = a;
+  }
+  __device__ static __forceinline__ float to_float(f16 v) { return (float)v; }
+  __device__ static __forceinline__ f16 from_float(float v) { return (f16)v; }
+  __device__ static __forceinline__ float init_lo() { return __builtin_inff(); }  // half(1e30) is +inf
+  __device__ static __forceinline__ float init_hi() { return -__builtin_inff(); }
+  // range is a half operation; the quotient is a double narrowed to float and then to half
+  __device__ static __forceinline__ f16 make_scale(f16 lo, f16 hi, int qmax) {
+    f16 range = hi - lo;
+    return (f16)(float)((double)(float)qmax / ((double)(float)range + 2e-6));
+  }
+  // half subtraction and half product (each rounded to half), then float from there on
+  __device__ static __forceinline__ int code(f16 x, f16 mn, f16 s, float u) {
+    f16 t = x - mn;
+    f16 p = t * s;
+    float y = (float)p + u;
+    float z = __builtin_fmaxf(y - 0.5f, 0.0f);
+    return (int)__builtin_rintf(z);
+  }
+  // half(code) / scale is a float division rounded to half; the sum is rounded to half again
+  __device__ static __forceinline__ f16 decode(int c, f16 s, f16 mn) {
+    f16 q = (f16)((float)c / (float)s);
+    return q + mn;
+  }
+};
+
+// Column of element e (0..7) of chunk k (0,1) for row lane i.
+__device__ __forceinline__ int chunk_col(int k, int i) { return 128 * k + 8 * i; }
+
+// Load the 16 elements lane i owns of group n; elements at or beyond numel read as zero (the zero
+// padding of gact/gact/ops.py:12-17 without the copy).
+template <typename T>
+__device__ __forceinline__ void load_group(const T* __restrict__ x, int64_t numel, int64_t n, int i,
+                                           T (&v)[2][8]) {
+  const int64_t base = n * GROUP;
+  if (base + GROUP <= numel) {
+#pragma unroll
+    for (int k = 0; k < 2; k++) Elem<T>::load8(x + base + chunk_col(k, i), v[k]);
+  } else {
+#pragma unroll
+    for (int k = 0; k < 2; k++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        int64_t idx = base + chunk_col(k, i) + e;
+        v[k][e] = idx < numel ? x[idx] : (T)0;
+      }
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ void store_group(T* __restrict__ out, int64_t numel, int64_t n, int i,
+                                            const T (&v)[2][8]) {
+  const int64_t base = n * GROUP;
+  if (base + GROUP <= numel) {
+#pragma unroll
+    for (int k = 0; k < 2; k++) Elem<T>::store8(out + base + chunk_col(k, i), v[k]);
+  } else {
+#pragma unroll
+    for (int k = 0; k < 2; k++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        int64_t idx = base + chunk_col(k, i) + e;
+        if (idx < numel) out[idx] = v[k][e];
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Quantize: the 8 groups of one row.
+//   GIVEN = false: min/max are reduced here (fused minimax + scale + pack, one read of x).
+//   GIVEN = true : min/max are read from mn_io / mx_io (the pack entry point's contract).
+// Codes follow quantization_cuda_kernel.cu:38-71; see Elem<T>::code for the arithmetic.
+// ------------------------------------------------------------------------------------------------
+template <typename T, int BITS, int NOISE, bool GIVEN>
+__device__ __forceinline__ void quantize_row(const T* __restrict__ x, int64_t numel, int64_t N, int64_t row,
+                                             int i, uint8_t* __restrict__ packed, T* __restrict__ scale_out,
+                                             T* mn_io, T* mx_io, uint64_t seed,
+                                             const float* __restrict__ noise) {
+  constexpr int WPT = 8 / BITS;
+  constexpr int QMAX = (1 << BITS) - 1;
+  const uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+
+#pragma unroll 1
+  for (int it = 0; it < BITS; it++) {  // BITS super-groups of WPT groups = 8 groups
+    const int64_t sg = row * BITS + it;
+    const int64_t n0 = sg * WPT;
+    if (n0 >= N) break;
+
+    T v[WPT][2][8];
+    T lo_t[WPT], s_t[WPT];
+#pragma unroll
+    for (int ni = 0; ni < WPT; ni++) {
+      if (n0 + ni < N) load_group<T>(x, numel, n0 + ni, i, v[ni]);
+    }
+#pragma unroll
+    for (int ni = 0; ni < WPT; ni++) {
+      const int64_t n = n0 + ni;
+      if (n < N) {
+        T lo_v, hi_v;
+        if (GIVEN) {
+          lo_v = mn_io[n];
+          hi_v = mx_io[n];
+        } else {
+          float lo = Elem<T>::init_lo(), hi = Elem<T>::init_hi();
+#pragma unroll
+          for (int k = 0; k < 2; k++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+              float f = Elem<T>::to_float(v[ni][k][e]);
+              lo = __builtin_fminf(lo, f);
+              hi = __builtin_fmaxf(hi, f);
+            }
+          lo = row_all_min(lo);
+          hi = row_all_max(hi);
+          lo_v = Elem<T>::from_float(lo);
+          hi_v = Elem<T>::from_float(hi);
+        }
+        T s = Elem<T>::make_scale(lo_v, hi_v, QMAX);
+        lo_t[ni] = lo_v;
+        s_t[ni] = s;
+        if (i == ni) {
+          scale_out[n] = s;
+          if (!GIVEN) {
+            mn_io[n] = lo_v;
+            if (mx_io) mx_io[n] = hi_v;
+          }
+        }
+      }
+    }
+
+    uint32_t bytes[2][8];
+#pragma unroll
+    for (int k = 0; k < 2; k++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) bytes[k][e] = 0;
+
+    if (NOISE == GACT_NOISE_REF) {
+      // one Philox state per output byte j: key = seed, counter = (draw/4, 0, j lo, j hi)
+#pragma unroll
+      for (int k = 0; k < 2; k++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const uint64_t j = (uint64_t)sg * GROUP + chunk_col(k, i) + e;
+          uint32_t r[4];
+#pragma unroll
+          for (int ni = 0; ni < WPT; ni++) {
+            if ((ni & 3) == 0) philox4x32_10(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r);
+            if (n0 + ni < N) {
+              float u = curand_uniform_map(r[ni & 3]);
+              int c = Elem<T>::code(v[ni][k][e], lo_t[ni], s_t[ni], u);
+              bytes[k][e] |= (uint32_t)c << (ni * BITS);
+            }
+          }
+        }
+    } else {
+#pragma unroll
+      for (int ni = 0; ni < WPT; ni++) {
+        const int64_t n = n0 + ni;
+        if (n < N) {
+#pragma unroll
+          for (int k = 0; k < 2; k++) {
+            float u[8];
+            if (NOISE == GACT_NOISE_CONST) {
+#pragma unroll
+              for (int e = 0; e < 8; e++) u[e] = 0.5f;
+            } else if (NOISE == GACT_NOISE_INJECT) {
+              Elem<float>::load8(noise + n * GROUP + chunk_col(k, i), u);
+            } else {  // GACT_NOISE_FAST: block index = flat element index / 8
+              const uint64_t blk = (uint64_t)n * (GROUP / 8) + 16 * k + i;
+              uint32_t r[4];
+              philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
+#pragma unroll
+              for (int e = 0; e < 8; e++) u[e] = fast_uniform_map((e & 1) ? (r[e >> 1] >> 16) : (r[e >> 1] & 0xffffu));
+            }
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+              int c = Elem<T>::code(v[ni][k][e], lo_t[ni], s_t[ni], u[e]);
+              bytes[k][e] |= (uint32_t)c << (ni * BITS);
+            }
+          }
+        }
+      }
+    }
+
+    // the reference accumulates in a uint8_t: keep the low 8 bits of every byte, then 8 bytes per chunk
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+      u32x2 w;
+      w.x = (bytes[k][0] & 0xffu) | ((bytes[k][1] & 0xffu) << 8) | ((bytes[k][2] & 0xffu) << 16) | (bytes[k][3] << 24);
+      w.y = (bytes[k][4] & 0xffu) | ((bytes[k][5] & 0xffu) << 8) | ((bytes[k][6] & 0xffu) << 16) | (bytes[k][7] << 24);
+      *reinterpret_cast<u32x2*>(packed + sg * GROUP + chunk_col(k, i)) = w;
+    }
+  }
+}
+
+// Dequantize: the 8 groups of one row.  quantization_cuda_kernel.cu:149-177.
+template <typename T, int BITS>
+__device__ __forceinline__ void dequantize_row(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
+                                               const T* __restrict__ mn, int64_t numel, int64_t N, int64_t row,
+                                               int i, T* __restrict__ out) {
+  constexpr int WPT = 8 / BITS;
+#pragma unroll 1
+  for (int it = 0; it < BITS; it++) {
+    const int64_t sg = row * BITS + it;
+    const int64_t n0 = sg * WPT;
+    if (n0 >= N) break;
+    u32x2 w[2];
+#pragma unroll
+    for (int k = 0; k < 2; k++) w[k] = *reinterpret_cast<const u32x2*>(packed + sg * GROUP + chunk_col(k, i));
+#pragma unroll
+    for (int ni = 0; ni < WPT; ni++) {
+      const int64_t n = n0 + ni;
+      if (n < N) {
+        const T s = scale[n];
+        const T m = mn[n];
+        T v[2][8];
+#pragma unroll
+        for (int k = 0; k < 2; k++)
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            uint32_t word = (e < 4) ? w[k].x : w[k].y;
+            int c = (int)__builtin_amdgcn_ubfe(word, 8 * (e & 3) + ni * BITS, BITS);
+            v[k][e] = Elem<T>::decode(c, s, m);
+          }
+        store_group<T>(out, numel, n, i, v);
+      }
+    }
+  }
+}
+
+// Row min/max only (the minimax entry point at D = 256).
+template <typename T>
+__device__ __forceinline__ void minimax_row(const T* __restrict__ x, int64_t N, int64_t row, int i,
+                                            T* __restrict__ mn, T* __restrict__ mx) {
+#pragma unroll 2
+  for (int g = 0; g < ROW_GROUPS; g++) {
+    const int64_t n = row * ROW_GROUPS + g;
+    if (n >= N) break;
+    T v[2][8];
+    load_group<T>(x, N * GROUP, n, i, v);
+    float lo = Elem<T>::init_lo(), hi = Elem<T>::init_hi();
+#pragma unroll
+    for (int k = 0; k < 2; k++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        float f = Elem<T>::to_float(v[k][e]);
+        lo = __builtin_fminf(lo, f);
+        hi = __builtin_fmaxf(hi, f);
+      }
+    lo = row_all_min(lo);
+    hi = row_all_max(hi);
+    if (i == 0) {
+      mn[n] = Elem<T>::from_float(lo);
+      mx[n] = Elem<T>::from_float(hi);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Single-tensor kernels.
+// ------------------------------------------------------------------------------------------------
+template <typename T, int BITS, int NOISE, bool GIVEN>
+__global__ void __launch_bounds__(256)
+quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
+                T* __restrict__ scale_out, T* mn_io, T* mx_io, uint64_t seed, const float* __restrict__ noise) {
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
+  if (row * ROW_GROUPS >= N) return;
+  quantize_row<T, BITS, NOISE, GIVEN>(x, numel, N, row, threadIdx.x & 15, packed, scale_out, mn_io, mx_io, seed, noise);
+}
+
+template <typename T, int BITS>
+__global__ void __launch_bounds__(256)
+dequantize_kernel(const uint8_t* __restrict__ packed, const T* __restrict__ scale, const T* __restrict__ mn,
+                  int64_t numel, int64_t N, T* __restrict__ out) {
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
+  if (row * ROW_GROUPS >= N) return;
+  dequantize_row<T, BITS>(packed, scale, mn, numel, N, row, threadIdx.x & 15, out);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+minimax256_kernel(const T* __restrict__ x, int64_t N, T* __restrict__ mn, T* __restrict__ mx) {
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
+  if (row * ROW_GROUPS >= N) return;
+  minimax_row<T>(x, N, row, threadIdx.x & 15, mn, mx);
+}
+
+// ------------------------------------------------------------------------------------------------
+// General shapes (any D for minimax; any G, D for pack / unpack).  These keep the operator surface
+// complete; the path the library is built for is G = 1, D = 256 above.
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+minimax_any_kernel(const T* __restrict__ x, int64_t N, int64_t D, T* __restrict__ mn, T* __restrict__ mx) {
+  // one wave per row
+  const int64_t n = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (n >= N) return;
+  const int lane = threadIdx.x & 63;
+  float lo = Elem<T>::init_lo(), hi = Elem<T>::init_hi();
+  for (int64_t d = lane; d < D; d += 64) {
+    float f = Elem<T>::to_float(x[n * D + d]);
+    lo = __builtin_fminf(lo, f);
+    hi = __builtin_fmaxf(hi, f);
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    lo = __builtin_fminf(lo, __shfl_xor(lo, off, 64));
+    hi = __builtin_fmaxf(hi, __shfl_xor(hi, off, 64));
+  }
+  if (lane == 0) {
+    mn[n] = Elem<T>::from_float(lo);
+    mx[n] = Elem<T>::from_float(hi);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+scale_kernel(const T* __restrict__ mn, const T* __restrict__ mx, int bits, int64_t count, T* __restrict__ scale) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id < count) scale[id] = Elem<T>::make_scale(mn[id], mx[id], (1 << bits) - 1);
+}
+
+// one thread per output byte j = (no*G + g)*D + d
+template <typename T, int NOISE>
+__global__ void __launch_bounds__(256)
+pack_any_kernel(const T* __restrict__ data, const T* __restrict__ mn, const T* __restrict__ scale, int bits,
+                int64_t N, int64_t G, int64_t D, uint64_t seed, const float* __restrict__ noise,
+                uint8_t* __restrict__ packed, int64_t total_bytes) {
+  const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= total_bytes) return;
+  const int wpt = 8 / bits;
+  const int64_t d = j % D;
+  const int64_t g = (j / D) % G;
+  const int64_t no = j / (D * G);
+  const uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+  uint32_t r[4];
+  uint32_t byte = 0;
+  for (int ni = 0; ni < wpt; ni++) {
+    const int64_t n = no * wpt + ni;
+    if (n >= N) break;
+    const int64_t id = (n * G + g) * D + d;
+    const int64_t sid = n * G + g;
+    float u = 0.5f;
+    if (NOISE == GACT_NOISE_INJECT) {
+      u = noise[id];
+    } else if (NOISE == GACT_NOISE_REF) {
+      if ((ni & 3) == 0) philox4x32_10(ni >> 2, 0u, (uint32_t)j, (uint32_t)((uint64_t)j >> 32), k0, k1, r);
+      u = curand_uniform_map(r[ni & 3]);
+    } else if (NOISE == GACT_NOISE_FAST) {
+      const uint64_t blk = (uint64_t)id >> 3;
+      philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
+      const int e = (int)(id & 7);
+      u = fast_uniform_map((e & 1) ? (r[e >> 1] >> 16) : (r[e >> 1] & 0xffffu));
+    }
+    int c = Elem<T>::code(data[id], mn[sid], scale[sid], u);
+    byte |= (uint32_t)c << (ni * bits);
+  }
+  packed[j] = (uint8_t)byte;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+unpack_any_kernel(const uint8_t* __restrict__ packed, int bits, const T* __restrict__ scale,
+                  const T* __restrict__ mn, int64_t N, int64_t G, int64_t D, T* __restrict__ out,
+                  int64_t total_bytes) {
+  const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= total_bytes) return;
+  const int wpt = 8 / bits;
+  const int64_t d = j % D;
+  const int64_t g = (j / D) % G;
+  const int64_t no = j / (D * G);
+  const uint32_t byte = packed[j];
+  for (int ni = 0; ni < wpt; ni++) {
+    const int64_t n = no * wpt + ni;
+    if (n >= N) break;
+    const int64_t sid = n * G + g;
+    int c = (int)((byte >> (ni * bits)) & ((1u << bits) - 1u));
+    out[(n * G + g) * D + d] = Elem<T>::decode(c, scale[sid], mn[sid]);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Dropout-mask bit packing.  Within each 512-element block, element e = k*16 + w is bit k of word w
+// (quantization_cuda_kernel.cu:228-252): with one 16-byte load per lane, lane k holds elements
+// 16k .. 16k+15, so word w is the ballot over lanes of "byte w is nonzero"; one wave packs two blocks
+// (low and high half of each ballot).  A partial last block is packed sequentially (element e -> word
+// e/32, bit e%32), which is the plain ballot of one byte per lane and fits the ceil(n/32)-word output.
+// ------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+mask_pack_kernel(const uint8_t* __restrict__ data, int64_t n, int32_t* __restrict__ mask) {
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int64_t full_blocks = n / 512;
+  const int64_t blk0 = wave * 2;  // this wave packs blocks blk0 and blk0 + 1
+  if (blk0 < full_blocks) {
+    const bool have = (blk0 + (lane >> 5)) < full_blocks;
+    u32x4 q = {0u, 0u, 0u, 0u};
+    if (have) q = *reinterpret_cast<const u32x4*>(data + (blk0 * 32 + lane) * 16);
+    uint32_t mine = 0;
+#pragma unroll
+    for (int w = 0; w < 16; w++) {
+      const uint32_t word = w < 4 ? q.x : w < 8 ? q.y : w < 12 ? q.z : q.w;
+      const uint64_t b = __ballot(((word >> (8 * (w & 3))) & 0xffu) != 0u);
+      if ((lane & 15) == w) mine = (lane & 16) ? (uint32_t)(b >> 32) : (uint32_t)b;
+    }
+    if (lane < 32 && (blk0 + (lane >> 4)) < full_blocks) mask[blk0 * 16 + lane] = (int32_t)mine;
+  }
+  // the partial block goes to the wave after the last full pair
+  if (wave == (full_blocks + 1) / 2) {
+    const int64_t base = full_blocks * 512;
+    const int64_t words = (n + 31) / 32;
+    for (int64_t e0 = base; e0 < n; e0 += 64) {
+      const int64_t e = e0 + lane;
+      const uint64_t b = __ballot(e < n && data[e] != 0);
+      const int64_t w = full_blocks * 16 + (e0 - base) / 32;
+      if (lane == 0) mask[w] = (int32_t)(uint32_t)b;
+      if (lane == 1 && w + 1 < words) mask[w + 1] = (int32_t)(uint32_t)(b >> 32);
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256)
+mask_unpack_kernel(const int32_t* __restrict__ mask, int64_t n, uint8_t* __restrict__ out) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // 16 elements per thread
+  const int64_t full_blocks = n / 512;
+  const int64_t blk = t >> 5;
+  const int k = (int)(t & 31);
+  if (blk < full_blocks) {
+    uint32_t q[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int w = 0; w < 16; w++) {
+      const uint32_t bit = ((uint32_t)mask[blk * 16 + w] >> k) & 1u;
+      q[w >> 2] |= bit << (8 * (w & 3));
+    }
+    u32x4 v = {q[0], q[1], q[2], q[3]};
+    *reinterpret_cast<u32x4*>(out + t * 16) = v;
+  } else if (blk == full_blocks) {
+    const int64_t base = full_blocks * 512;
+    for (int64_t e = base + k * 16; e < base + k * 16 + 16 && e < n; e++) {
+      const int64_t r = e - base;
+      out[e] = (uint8_t)(((uint32_t)mask[full_blocks * 16 + r / 32] >> (r % 32)) & 1u);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Greedy bit allocation.  calc_precision.cc:66-118: a max-heap of (float key, index) compared
+// lexicographically; indices are distinct, so the pop order is the descending total order and an
+// argmax restates it.  Keys are doubles narrowed to float exactly as the heap's pair<float, int64> does.
+// ------------------------------------------------------------------------------------------------
+__host__ __device__ inline int prec_next_bits(int b) { return b == 32 ? 8 : b == 8 ? 4 : b == 4 ? 2 : b == 2 ? 1 : 0; }
+__host__ __device__ inline float prec_key(float C, int b, int64_t w) {
+  const int nb = prec_next_bits(b);
+  const int coeff_2 = ((1 << nb) - 1) * ((1 << nb) - 1);
+  double obj;
+  if (b == 32) {
+    obj = -(double)C / coeff_2;
+  } else {
+    const int coeff_1 = ((1 << b) - 1) * ((1 << b) - 1);
+    obj = C * (1.0 / coeff_1 - 1.0 / coeff_2);
+  }
+  return (float)(obj / (double)(w * (int64_t)(b - nb)));
+}
+__host__ __device__ inline bool prec_valid_bits(int b) { return b == 1 || b == 2 || b == 4 || b == 8 || b == 32; }
+
+#define PREC_MAX_L 4096
+__global__ void __launch_bounds__(64)
+calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, const int64_t* __restrict__ w,
+                      int L, double target, int32_t* __restrict__ status) {
+  __shared__ float key_s[PREC_MAX_L];
+  __shared__ int32_t b_s[PREC_MAX_L];
+  const int lane = threadIdx.x;
+  double part = 0.0;
+  for (int idx = lane; idx < L; idx += 64) {
+    const int bi = b[idx];
+    b_s[idx] = bi;
+    if (bi > 1) {
+      key_s[idx] = prec_key(C[idx], bi, w[idx]);
+      part += (double)((int64_t)bi * w[idx]);
+    }
+  }
+  // every term is an integer; the sum is exact (and order-free) below 2^53
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) part += __shfl_xor(part, off, 64);
+  double b_sum = part;
+  __syncthreads();
+  int rc = 0;
+  while (b_sum > target) {
+    float best_key = 0.0f;
+    int best = -1;
+    for (int idx = lane; idx < L; idx += 64) {
+      if (b_s[idx] > 1) {
+        const float k = key_s[idx];
+        if (best < 0 || best_key < k || (!(k < best_key) && idx > best)) { best_key = k; best = idx; }
+      }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      const float ok = __shfl_xor(best_key, off, 64);
+      const int oi = __shfl_xor(best, off, 64);
+      if (oi >= 0 && (best < 0 || best_key < ok || (!(ok < best_key) && oi > best))) { best_key = ok; best = oi; }
+    }
+    if (best < 0) { rc = GACT_EBUDGET; break; }
+    const int cur = b_s[best];
+    const int nb = prec_next_bits(cur);
+    const int64_t wb = w[best];
+    __syncthreads();
+    if (lane == 0) {
+      b_s[best] = nb;
+      if (nb > 1) key_s[best] = prec_key(C[best], nb, wb);
+    }
+    b_sum -= (double)(wb * (int64_t)(cur - nb));
+    __syncthreads();
+  }
+  for (int idx = lane; idx < L; idx += 64) b[idx] = b_s[idx];
+  if (status && lane == 0) *status = rc;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Batched launch over a table of tensors with device-resident bits.
+// ------------------------------------------------------------------------------------------------
+__global__ void batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int L,
+                                  int64_t* total) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  int64_t off = 0;
+  for (int t = 0; t < L; t++) {
+    const int bt = bits[t];
+    const int wpt = 8 / (bt > 0 && bt <= 8 ? bt : 8);
+    const int64_t N = (table[t].numel + GROUP - 1) / GROUP;
+    const int64_t n_round = (N + wpt - 1) / wpt * wpt;
+    table[t].packed_offset = off;
+    off += ((int64_t)bt * n_round * (GROUP / 8) + 255) / 256 * 256;
+  }
+  if (total) *total = off;
+}
+
+__device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ table, int L, int64_t block) {
+  int lo = 0, hi = L - 1;  // last entry with first_block <= block
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (table[mid].first_block <= block) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+template <int NOISE>
+__global__ void __launch_bounds__(256)
+quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
+                        uint8_t* __restrict__ packed_arena, uint8_t* __restrict__ scale_arena,
+                        uint8_t* __restrict__ min_arena) {
+  const int t = batch_find(table, L, blockIdx.x);
+  const gact_batch_entry ent = table[t];
+  const int bt = bits[t];
+  const int64_t N = (ent.numel + GROUP - 1) / GROUP;
+  const int64_t row = ((int64_t)blockIdx.x - ent.first_block) * 16 + (threadIdx.x >> 4);
+  if (row * ROW_GROUPS >= N) return;
+  const int i = threadIdx.x & 15;
+  uint8_t* packed = packed_arena + ent.packed_offset;
+  uint8_t* sc = scale_arena + ent.stats_offset * 4;
+  uint8_t* mn = min_arena + ent.stats_offset * 4;
+#define GACT_QB(T, B) \
+  quantize_row<T, B, NOISE, false>((const T*)ent.x, ent.numel, N, row, i, packed, (T*)sc, (T*)mn, (T*)nullptr, ent.seed, nullptr)
+  if (ent.dtype == GACT_F32) {
+    switch (bt) {
+      case 1: GACT_QB(float, 1); break;
+      case 2: GACT_QB(float, 2); break;
+      case 4: GACT_QB(float, 4); break;
+      case 8: GACT_QB(float, 8); break;
+    }
+  } else {
+    switch (bt) {
+      case 1: GACT_QB(f16, 1); break;
+      case 2: GACT_QB(f16, 2); break;
+      case 4: GACT_QB(f16, 4); break;
+      case 8: GACT_QB(f16, 8); break;
+    }
+  }
+#undef GACT_QB
+}
+
+__global__ void __launch_bounds__(256)
+dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
+                          const uint8_t* __restrict__ packed_arena, const uint8_t* __restrict__ scale_arena,
+                          const uint8_t* __restrict__ min_arena) {
+  const int t = batch_find(table, L, blockIdx.x);
+  const gact_batch_entry ent = table[t];
+  const int bt = bits[t];
+  const int64_t N = (ent.numel + GROUP - 1) / GROUP;
+  const int64_t row = ((int64_t)blockIdx.x - ent.first_block) * 16 + (threadIdx.x >> 4);
+  if (row * ROW_GROUPS >= N) return;
+  const int i = threadIdx.x & 15;
+  const uint8_t* packed = packed_arena + ent.packed_offset;
+  const uint8_t* sc = scale_arena + ent.stats_offset * 4;
+  const uint8_t* mn = min_arena + ent.stats_offset * 4;
+#define GACT_DB(T, B) dequantize_row<T, B>(packed, (const T*)sc, (const T*)mn, ent.numel, N, row, i, (T*)ent.x)
+  if (ent.dtype == GACT_F32) {
+    switch (bt) {
+      case 1: GACT_DB(float, 1); break;
+      case 2: GACT_DB(float, 2); break;
+      case 4: GACT_DB(float, 4); break;
+      case 8: GACT_DB(float, 8); break;
+    }
+  } else {
+    switch (bt) {
+      case 1: GACT_DB(f16, 1); break;
+      case 2: GACT_DB(f16, 2); break;
+      case 4: GACT_DB(f16, 4); break;
+      case 8: GACT_DB(f16, 8); break;
+    }
+  }
+#undef GACT_DB
+}
+
+// ------------------------------------------------------------------------------------------------
+// Host side of the C ABI.
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+inline bool valid_bits(int bits) { return bits == 1 || bits == 2 || bits == 4 || bits == 8; }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int launch_status() { return hipGetLastError() == hipSuccess ? GACT_OK : GACT_ELAUNCH; }
+
+// rows of 8 groups; 16 rows per 256-thread block, or 4 rows per 64-thread block when the tensor is
+// too small to give every CU a block otherwise
+inline void row_grid(int64_t N, dim3* grid, dim3* block) {
+  const int64_t rows = (N + ROW_GROUPS - 1) / ROW_GROUPS;
+  int threads = 256;
+  if ((rows + 15) / 16 < 2048) threads = 64;
+  const int rows_per_block = threads / 16;
+  *grid = dim3((unsigned)((rows + rows_per_block - 1) / rows_per_block));
+  *block = dim3(threads);
+}
+
+template <typename T, int BITS, bool GIVEN>
+int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, T* scale, T* mn, T* mx, int noise_mode,
+                    uint64_t seed, const float* noise, hipStream_t stream) {
+  dim3 grid, block;
+  row_grid(N, &grid, &block);
+  switch (noise_mode) {
+    case GACT_NOISE_CONST:
+      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_CONST, GIVEN>), grid, block, 0, stream, x, numel, N,
+                         packed, scale, mn, mx, seed, noise);
+      break;
+    case GACT_NOISE_INJECT:
+      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_INJECT, GIVEN>), grid, block, 0, stream, x, numel, N,
+                         packed, scale, mn, mx, seed, noise);
+      break;
+    case GACT_NOISE_REF:
+      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_REF, GIVEN>), grid, block, 0, stream, x, numel, N,
+                         packed, scale, mn, mx, seed, noise);
+      break;
+    case GACT_NOISE_FAST:
+      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_FAST, GIVEN>), grid, block, 0, stream, x, numel, N,
+                         packed, scale, mn, mx, seed, noise);
+      break;
+    default:
+      return GACT_EINVAL;
+  }
+  return launch_status();
+}
+
+template <typename T, bool GIVEN>
+int dispatch_quantize(int bits, const T* x, int64_t numel, int64_t N, uint8_t* packed, T* scale, T* mn, T* mx,
+                      int noise_mode, uint64_t seed, const float* noise, hipStream_t stream) {
+  switch (bits) {
+    case 1: return launch_quantize<T, 1, GIVEN>(x, numel, N, packed, scale, mn, mx, noise_mode, seed, noise, stream);
+    case 2: return launch_quantize<T, 2, GIVEN>(x, numel, N, packed, scale, mn, mx, noise_mode, seed, noise, stream);
+    case 4: return launch_quantize<T, 4, GIVEN>(x, numel, N, packed, scale, mn, mx, noise_mode, seed, noise, stream);
+    case 8: return launch_quantize<T, 8, GIVEN>(x, numel, N, packed, scale, mn, mx, noise_mode, seed, noise, stream);
+  }
+  return GACT_EINVAL;
+}
+
+template <typename T>
+int dispatch_dequantize(int bits, const uint8_t* packed, const T* scale, const T* mn, int64_t numel, int64_t N, T* out,
+                        hipStream_t stream) {
+  dim3 grid, block;
+  row_grid(N, &grid, &block);
+  switch (bits) {
+    case 1: hipLaunchKernelGGL((dequantize_kernel<T, 1>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
+    case 2: hipLaunchKernelGGL((dequantize_kernel<T, 2>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
+    case 4: hipLaunchKernelGGL((dequantize_kernel<T, 4>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
+    case 8: hipLaunchKernelGGL((dequantize_kernel<T, 8>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
+    default: return GACT_EINVAL;
+  }
+  return launch_status();
+}
+
+template <typename T>
+int pack_any(const T* data, const T* mn, const T* scale, int bits, int64_t N, int64_t G, int64_t D, int noise_mode,
+             uint64_t seed, const float* noise, uint8_t* packed, hipStream_t stream) {
+  const int64_t total = gact_packed_bytes(bits, N, G, D);
+  const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  switch (noise_mode) {
+    case GACT_NOISE_CONST:
+      hipLaunchKernelGGL((pack_any_kernel<T, GACT_NOISE_CONST>), grid, block, 0, stream, data, mn, scale, bits, N, G, D, seed, noise, packed, total);
+      break;
+    case GACT_NOISE_INJECT:
+      hipLaunchKernelGGL((pack_any_kernel<T, GACT_NOISE_INJECT>), grid, block, 0, stream, data, mn, scale, bits, N, G, D, seed, noise, packed, total);
+      break;
+    case GACT_NOISE_REF:
+      hipLaunchKernelGGL((pack_any_kernel<T, GACT_NOISE_REF>), grid, block, 0, stream, data, mn, scale, bits, N, G, D, seed, noise, packed, total);
+      break;
+    case GACT_NOISE_FAST:
+      hipLaunchKernelGGL((pack_any_kernel<T, GACT_NOISE_FAST>), grid, block, 0, stream, data, mn, scale, bits, N, G, D, seed, noise, packed, total);
+      break;
+    default:
+      return GACT_EINVAL;
+  }
+  return launch_status();
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* gact_strerror(int code) {
+  switch (code) {
+    case GACT_OK: return "ok";
+    case GACT_EINVAL: return "invalid argument";
+    case GACT_EALIGN: return "pointer is not 16-byte aligned";
+    case GACT_ESHAPE: return "unsupported shape";
+    case GACT_ELAUNCH: return "HIP launch failed";
+    case GACT_EBUDGET: return "bit budget unreachable: every tensor is already at 1 bit";
+  }
+  return "unknown error";
+}
+
+int gact_abi_version(void) { return GACT_ABI_VERSION; }
+
+int64_t gact_packed_bytes(int bits, int64_t N, int64_t G, int64_t D) {
+  if (!valid_bits(bits) || N < 0 || G < 0 || D < 0) return GACT_EINVAL;
+  const int wpt = 8 / bits;
+  const int64_t n_round = (N + wpt - 1) / wpt * wpt;
+  return (int64_t)bits * n_round * G * D / 8;
+}
+
+int gact_minimax(const void* data, int dtype, int64_t N, int64_t D, void* mn, void* mx, void* stream) {
+  if (dtype != GACT_F32 && dtype != GACT_F16) return GACT_EINVAL;
+  if (N < 0 || !(D % 32 == 0 && D > 32)) return GACT_ESHAPE;  // minimax_cuda_kernel.cu:80
+  if (N == 0) return GACT_OK;
+  if (!data || !mn || !mx) return GACT_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  if (D == GROUP && aligned16(data)) {
+    dim3 grid, block;
+    row_grid(N, &grid, &block);
+    if (dtype == GACT_F32)
+      hipLaunchKernelGGL((minimax256_kernel<float>), grid, block, 0, s, (const float*)data, N, (float*)mn, (float*)mx);
+    else
+      hipLaunchKernelGGL((minimax256_kernel<f16>), grid, block, 0, s, (const f16*)data, N, (f16*)mn, (f16*)mx);
+  } else {
+    const dim3 grid((unsigned)((N + 3) / 4)), block(256);
+    if (dtype == GACT_F32)
+      hipLaunchKernelGGL((minimax_any_kernel<float>), grid, block, 0, s, (const float*)data, N, D, (float*)mn, (float*)mx);
+    else
+      hipLaunchKernelGGL((minimax_any_kernel<f16>), grid, block, 0, s, (const f16*)data, N, D, (f16*)mn, (f16*)mx);
+  }
+  return launch_status();
+}
+
+int gact_pack(const void* data, const void* mn, const void* mx, int dtype, int bits, int64_t N, int64_t G, int64_t D,
+              int noise_mode, uint64_t seed, const float* noise, void* packed, void* scale, void* stream) {
+  if (dtype != GACT_F32 && dtype != GACT_F16) return GACT_EINVAL;
+  if (!valid_bits(bits)) return GACT_EINVAL;  // quantization_cuda_kernel.cu:86
+  if (N < 0 || G < 0 || D < 0) return GACT_EINVAL;
+  if (noise_mode < GACT_NOISE_CONST || noise_mode > GACT_NOISE_FAST) return GACT_EINVAL;
+  if (N * G * D == 0) return GACT_OK;
+  if (!data || !mn || !mx || !packed || !scale) return GACT_EINVAL;
+  if (noise_mode == GACT_NOISE_INJECT && !noise) return GACT_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  if (G == 1 && D == GROUP && aligned16(data) && aligned16(packed) && (noise_mode != GACT_NOISE_INJECT || aligned16(noise))) {
+    // the fused row kernel with min/max taken from the caller
+    if (dtype == GACT_F32)
+      return dispatch_quantize<float, true>(bits, (const float*)data, N * GROUP, N, (uint8_t*)packed, (float*)scale,
+                                            (float*)const_cast<void*>(mn), (float*)const_cast<void*>(mx), noise_mode, seed, noise, s);
+    return dispatch_quantize<f16, true>(bits, (const f16*)data, N * GROUP, N, (uint8_t*)packed, (f16*)scale,
+                                        (f16*)const_cast<void*>(mn), (f16*)const_cast<void*>(mx), noise_mode, seed, noise, s);
+  }
+  const int64_t count = N * G;
+  const dim3 sgrid((unsigned)((count + 255) / 256)), sblock(256);
+  if (dtype == GACT_F32) {
+    hipLaunchKernelGGL((scale_kernel<float>), sgrid, sblock, 0, s, (const float*)mn, (const float*)mx, bits, count, (float*)scale);
+    return pack_any<float>((const float*)data, (const float*)mn, (const float*)scale, bits, N, G, D, noise_mode, seed, noise, (uint8_t*)packed, s);
+  }
+  hipLaunchKernelGGL((scale_kernel<f16>), sgrid, sblock, 0, s, (const f16*)mn, (const f16*)mx, bits, count, (f16*)scale);
+  return pack_any<f16>((const f16*)data, (const f16*)mn, (const f16*)scale, bits, N, G, D, noise_mode, seed, noise, (uint8_t*)packed, s);
+}
+
+int gact_unpack(const void* packed, int bits, const void* scale, const void* mn, int dtype, int64_t N, int64_t G,
+                int64_t D, void* out, void* stream) {
+  if (dtype != GACT_F32 && dtype != GACT_F16) return GACT_EINVAL;
+  if (!valid_bits(bits)) return GACT_EINVAL;  // quantization_cuda_kernel.cu:191
+  if (N < 0 || G < 0 || D < 0) return GACT_EINVAL;
+  if (N * G * D == 0) return GACT_OK;
+  if (!packed || !scale || !mn || !out) return GACT_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  if (G == 1 && D == GROUP && aligned16(out) && aligned16(packed)) {
+    if (dtype == GACT_F32)
+      return dispatch_dequantize<float>(bits, (const uint8_t*)packed, (const float*)scale, (const float*)mn, N * GROUP, N, (float*)out, s);
+    return dispatch_dequantize<f16>(bits, (const uint8_t*)packed, (const f16*)scale, (const f16*)mn, N * GROUP, N, (f16*)out, s);
+  }
+  const int64_t total = gact_packed_bytes(bits, N, G, D);
+  const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  if (dtype == GACT_F32)
+    hipLaunchKernelGGL((unpack_any_kernel<float>), grid, block, 0, s, (const uint8_t*)packed, bits, (const float*)scale, (const float*)mn, N, G, D, (float*)out, total);
+  else
+    hipLaunchKernelGGL((unpack_any_kernel<f16>), grid, block, 0, s, (const uint8_t*)packed, bits, (const f16*)scale, (const f16*)mn, N, G, D, (f16*)out, total);
+  return launch_status();
+}
+
+int gact_quantize(const void* x, int dtype, int64_t numel, int bits, int noise_mode, uint64_t seed, const float* noise,
+                  void* packed, void* scale, void* mn, void* mx, void* stream) {
+  if (dtype != GACT_F32 && dtype != GACT_F16) return GACT_EINVAL;
+  if (!valid_bits(bits) || numel < 0) return GACT_EINVAL;
+  if (noise_mode < GACT_NOISE_CONST || noise_mode > GACT_NOISE_FAST) return GACT_EINVAL;
+  if (numel == 0) return GACT_OK;
+  if (!x || !packed || !scale || !mn) return GACT_EINVAL;
+  if (noise_mode == GACT_NOISE_INJECT && !noise) return GACT_EINVAL;
+  if (!aligned16(x) || !aligned16(packed) || (noise_mode == GACT_NOISE_INJECT && !aligned16(noise))) return GACT_EALIGN;
+  const int64_t N = (numel + GROUP - 1) / GROUP;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == GACT_F32)
+    return dispatch_quantize<float, false>(bits, (const float*)x, numel, N, (uint8_t*)packed, (float*)scale, (float*)mn, (float*)mx, noise_mode, seed, noise, s);
+  return dispatch_quantize<f16, false>(bits, (const f16*)x, numel, N, (uint8_t*)packed, (f16*)scale, (f16*)mn, (f16*)mx, noise_mode, seed, noise, s);
+}
+
+int gact_dequantize(const void* packed, int bits, const void* scale, const void* mn, int dtype, int64_t numel, void* out,
+                    void* stream) {
+  if (dtype != GACT_F32 && dtype != GACT_F16) return GACT_EINVAL;
+  if (!valid_bits(bits) || numel < 0) return GACT_EINVAL;
+  if (numel == 0) return GACT_OK;
+  if (!packed || !scale || !mn || !out) return GACT_EINVAL;
+  if (!aligned16(out) || !aligned16(packed)) return GACT_EALIGN;
+  const int64_t N = (numel + GROUP - 1) / GROUP;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == GACT_F32)
+    return dispatch_dequantize<float>(bits, (const uint8_t*)packed, (const float*)scale, (const float*)mn, numel, N, (float*)out, s);
+  return dispatch_dequantize<f16>(bits, (const uint8_t*)packed, (const f16*)scale, (const f16*)mn, numel, N, (f16*)out, s);
+}
+
+int gact_mask_pack(const uint8_t* data, int64_t n, int32_t* mask, void* stream) {
+  if (n < 0) return GACT_EINVAL;
+  if (n == 0) return GACT_OK;
+  if (!data || !mask) return GACT_EINVAL;
+  if (!aligned16(data)) return GACT_EALIGN;
+  const int64_t full_blocks = n / 512;
+  const int64_t waves = (full_blocks + 1) / 2 + 1;  // pairs of full blocks, plus the one that takes the partial block
+  hipLaunchKernelGGL(mask_pack_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, (hipStream_t)stream, data, n, mask);
+  return launch_status();
+}
+
+int gact_mask_unpack(const int32_t* mask, int64_t n, uint8_t* out, void* stream) {
+  if (n < 0) return GACT_EINVAL;
+  if (n == 0) return GACT_OK;
+  if (!mask || !out) return GACT_EINVAL;
+  if (!aligned16(out)) return GACT_EALIGN;
+  const int64_t threads = (n / 512 + 1) * 32;
+  hipLaunchKernelGGL(mask_unpack_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, (hipStream_t)stream, mask, n, out);
+  return launch_status();
+}
+
+int gact_calc_precision(int32_t* b, const float* C, const int64_t* w, int64_t L, double target) {
+  if (L < 0) return GACT_EINVAL;
+  if (L == 0) return GACT_OK;
+  if (!b || !C || !w) return GACT_EINVAL;
+  for (int64_t i = 0; i < L; i++)
+    if (!prec_valid_bits(b[i])) return GACT_EINVAL;
+  std::priority_queue<std::pair<float, int64_t>> q;
+  double b_sum = 0;
+  for (int64_t i = 0; i < L; i++)
+    if (b[i] > 1) {
+      q.push(std::make_pair(prec_key(C[i], b[i], w[i]), i));
+      b_sum += (double)((int64_t)b[i] * w[i]);
+    }
+  while (b_sum > target) {
+    if (q.empty()) return GACT_EBUDGET;
+    const int64_t i = q.top().second;
+    q.pop();
+    const int nb = prec_next_bits(b[i]);
+    b_sum -= (double)(w[i] * (int64_t)(b[i] - nb));
+    b[i] = nb;
+    if (nb > 1) q.push(std::make_pair(prec_key(C[i], nb, w[i]), i));
+  }
+  return GACT_OK;
+}
+
+int gact_calc_precision_device(int32_t* b, const float* C, const int64_t* w, int64_t L, double target, int32_t* status,
+                               void* stream) {
+  if (L < 0) return GACT_EINVAL;
+  if (L > PREC_MAX_L) return GACT_ESHAPE;
+  if (L == 0) return GACT_OK;
+  if (!b || !C || !w) return GACT_EINVAL;
+  hipLaunchKernelGGL(calc_precision_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, b, C, w, (int)L, target, status);
+  return launch_status();
+}
+
+int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t* total, void* stream) {
+  if (L < 0 || L > (1 << 30)) return GACT_EINVAL;
+  if (L == 0) return GACT_OK;
+  if (!table || !bits) return GACT_EINVAL;
+  hipLaunchKernelGGL(batch_plan_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, table, bits, (int)L, total);
+  return launch_status();
+}
+
+int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
+                          int noise_mode, void* packed_arena, void* scale_arena, void* min_arena, void* stream) {
+  if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x7fffffffLL) return GACT_EINVAL;
+  if (L == 0 || total_blocks == 0) return GACT_OK;
+  if (!table || !bits || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
+  if (!aligned16(packed_arena)) return GACT_EALIGN;
+  const dim3 grid((unsigned)total_blocks), block(256);
+  hipStream_t s = (hipStream_t)stream;
+  switch (noise_mode) {
+    case GACT_NOISE_CONST:
+      hipLaunchKernelGGL((quantize_batched_kernel<GACT_NOISE_CONST>), grid, block, 0, s, table, bits, (int)L, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena);
+      break;
+    case GACT_NOISE_REF:
+      hipLaunchKernelGGL((quantize_batched_kernel<GACT_NOISE_REF>), grid, block, 0, s, table, bits, (int)L, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena);
+      break;
+    case GACT_NOISE_FAST:
+      hipLaunchKernelGGL((quantize_batched_kernel<GACT_NOISE_FAST>), grid, block, 0, s, table, bits, (int)L, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena);
+      break;
+    default:
+      return GACT_EINVAL;  // injected noise is a single-tensor test mode
+  }
+  return launch_status();
+}
+
+int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
+                            const void* packed_arena, const void* scale_arena, const void* min_arena, void* stream) {
+  if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x7fffffffLL) return GACT_EINVAL;
+  if (L == 0 || total_blocks == 0) return GACT_OK;
+  if (!table || !bits || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
+  if (!aligned16(packed_arena)) return GACT_EALIGN;
+  hipLaunchKernelGGL(dequantize_batched_kernel, dim3((unsigned)total_blocks), dim3(256), 0, (hipStream_t)stream, table, bits, (int)L,
+                     (const uint8_t*)packed_arena, (const uint8_t*)scale_arena, (const uint8_t*)min_arena);
+  return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,82 @@
+"""Global configuration of the activation-compression path.
+
+Field names, defaults and optimisation levels follow gact/gact/conf.py:1-72 of the reference;
+``rng_stream`` is the one addition.
+"""
+
+
+class QuantizationConfig:
+    def __init__(self):
+        # compress activations; False at optimisation level L0
+        self.compress_activation = True
+
+        # ---- general quantisation ----
+        # average bits per activation element; with auto precision off every tensor uses this width
+        self.bit = 4
+        self.group_size = 256
+        # skip tensors that were already saved in this iteration (keyed by sampled contents)
+        self.check_dup = False
+
+        # ---- auto precision ----
+        self.auto_prec = True
+        self.max_bit = 32          # widest allocation the greedy search starts from
+        self.adapt_interval = 1000  # iterations between sensitivity refreshes
+        self.work_dir = "./log/"
+        self.log_interval = -1      # < 0 disables logging
+        self.debug = False
+
+        # ---- memory management ----
+        self.swap = False
+        self.prefetch = False
+
+        # ---- stochastic-rounding noise (not in the reference) ----
+        # "fast":          one Philox4x32-10 block per 8 elements, 16-bit uniforms
+        # "reference":     the reference's stream (one Philox state per output byte, cuRAND uniform map)
+        # "deterministic": u = 0.5 everywhere, i.e. round to nearest
+        self.rng_stream = "fast"
+
+
+config = QuantizationConfig()
+
+
+def set_optimization_level(level):
+    """gact/gact/conf.py:1-36."""
+    if level == 'L0':
+        config.compress_activation = False
+    elif level == 'L1':      # fixed 4 bit
+        config.auto_prec = False
+        config.bit = 4
+    elif level == 'L1.1':    # fixed 8 bit
+        config.auto_prec = False
+        config.bit = 8
+    elif level == 'L1.2':    # fixed 2 bit
+        config.auto_prec = False
+        config.bit = 2
+    elif level == 'L2':      # auto precision, 4 bit average
+        config.auto_prec = True
+        config.bit = 4
+    elif level == 'L2.1':    # auto precision, 3 bit average
+        config.auto_prec = True
+        config.bit = 3
+    elif level == 'L2.2':    # auto precision, 2 bit average
+        config.auto_prec = True
+        config.bit = 2
+    elif level == 'L3':      # auto precision 4 bit + swap
+        config.auto_prec = True
+        config.bit = 4
+        config.swap = True
+        config.prefetch = True
+    elif level == 'swap':    # swap only
+        config.swap = True
+        config.compress_activation = False
+    elif level == 'L4bit-swap':
+        config.bit = 4
+        config.swap = True
+        config.prefetch = True
+        config.auto_prec = False
+    else:
+        raise ValueError("Invalid level: " + level)
+
+
+def set_adapt_interval(i):
+    config.adapt_interval = i

@@ -1,0 +1,127 @@
+"""Quantize / dequantize operators with the reference's names and return conventions
+(gact/gact/ops.py:11-69), running on the fused HIP kernels.
+
+``op_quantize`` reads the activation once: min/max, scale, stochastic rounding and packing happen in a
+single kernel, and the zero padding to whole groups of 256 is done by the kernel's bounds handling
+instead of a concatenated copy.  ``op_dequantize`` writes straight into a tensor of the original
+shape.  The extension-style entry points (minimax, pack_single_precision, unpack_single_precision)
+stay available in gact.cpp_extension for callers that use them directly.
+"""
+import numpy as np
+import torch
+
+from .conf import config
+from .cpp_extension import _abi
+from .cpp_extension import quantization as ext_quantization
+
+
+def _num_groups(numel):
+    return (numel + config.group_size - 1) // config.group_size
+
+
+def _require_group_256():
+    if config.group_size != _abi.GROUP:
+        raise RuntimeError("the fused kernels are built for group_size 256, got %d" % config.group_size)
+
+
+def no_scheme_quantize_pack(input, q_bit, seed, *, noise=None, rng_stream=None):
+    """gact/gact/ops.py:11-32 -> (q_input, q_scale, q_min)."""
+    N = _num_groups(input.numel())
+    if q_bit == 32:
+        # the passthrough of ops.py:21-24: the padded [N, group] view itself, max - min, min
+        num_ele = N * config.group_size
+        pad_num = num_ele - input.numel()
+        if pad_num > 0:
+            input = torch.cat([input.reshape(1, -1),
+                               torch.zeros([1, pad_num], dtype=input.dtype, device=input.device)], dim=1)
+        input_groups = input.reshape(-1, config.group_size)
+        q_min = input_groups.min(dim=-1, keepdim=True).values
+        q_scale = input_groups.max(dim=-1, keepdim=True).values - q_min
+        return input_groups, q_scale, q_min
+
+    _require_group_256()
+    if not input.is_cuda:
+        raise RuntimeError("data must be a CUDA tensor!")
+    if input.dtype not in (torch.float32, torch.float16):
+        raise RuntimeError("The type of data is not correct!")
+    ext_quantization._check_bits(q_bit)
+    seed = ext_quantization._seed_u64(seed)
+    x = input.contiguous()  # the reference's reshape copies a non-contiguous input as well
+    if not _abi.aligned(x):
+        x = x.clone()
+    mode = ext_quantization._noise_mode(noise, rng_stream)
+    if noise is not None:
+        if (not noise.is_cuda) or noise.dtype != torch.float32 or noise.numel() != N * config.group_size \
+                or not noise.is_contiguous():
+            raise RuntimeError("noise must be a contiguous float32 CUDA tensor with one value per padded element")
+    q_input = torch.empty((ext_quantization.packed_numel(q_bit, N, 1, config.group_size),),
+                          dtype=torch.int8, device=x.device)
+    q_scale = torch.empty((N, 1, 1), dtype=x.dtype, device=x.device)
+    q_min = torch.empty((N, 1, 1), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _abi.check(_abi.lib().gact_quantize(x.data_ptr(), _abi.dtype_code(x.dtype), x.numel(), q_bit, mode, seed,
+                                            _abi.ptr(noise), q_input.data_ptr(), q_scale.data_ptr(),
+                                            q_min.data_ptr(), None, _abi.stream_of(x)))
+    return q_input, q_scale, q_min
+
+
+def dequantize_and_unpack(data, shape, q_bit, scale, mn):
+    """gact/gact/ops.py:34-47 -> [num_groups, 1, group_size] tensor (the padded groups)."""
+    if not isinstance(q_bit, int):
+        print("bits must be intergers, now bits ", q_bit)
+        assert(False)
+
+    if q_bit == 32:
+        return data
+
+    group_size = config.group_size
+    num_groups = (int(np.prod(shape)) + group_size - 1) // group_size
+    return ext_quantization.unpack_single_precision(data, q_bit, scale, mn, num_groups, 1, group_size)
+
+
+def op_quantize_mask(input):
+    """gact/gact/ops.py:49-50."""
+    return [ext_quantization.act_quantize_dropout_mask(input.contiguous()), input.shape]
+
+
+def op_dequantize_mask(input):
+    """gact/gact/ops.py:52-55."""
+    q_mask, input_shape = input
+    output = ext_quantization.act_dequantize_dropout_mask(q_mask, np.prod(input_shape)).reshape(input_shape)
+    return output
+
+
+def op_quantize(input, q_bit, seed, *, noise=None, rng_stream=None):
+    """gact/gact/ops.py:57-59 -> [q_input, q_bit, q_scale, q_min]."""
+    q_input, q_scale, q_min = no_scheme_quantize_pack(input, q_bit, seed, noise=noise, rng_stream=rng_stream)
+    return [q_input, q_bit, q_scale, q_min]
+
+
+def op_dequantize(input, input_shape):
+    """gact/gact/ops.py:61-69 -> tensor of `input_shape`, contiguous, dtype of the scale."""
+    q_input, q_bit, q_scale, q_min = input
+    if not isinstance(q_bit, int):
+        print("bits must be intergers, now bits ", q_bit)
+        assert(False)
+    num_features = int(np.prod(input_shape))
+    if q_bit == 32:
+        return q_input.ravel()[:num_features].reshape(*input_shape).contiguous()
+
+    _require_group_256()
+    ext_quantization._check_bits(q_bit)
+    if not q_input.is_cuda:
+        raise RuntimeError("data must be a CUDA tensor!")
+    if q_input.dtype != torch.int8 or q_input.dim() != 1:
+        raise RuntimeError("The type of data is not correct!")
+    N = _num_groups(num_features)
+    if q_input.numel() < ext_quantization.packed_numel(q_bit, N, 1, config.group_size) - 1 \
+            or q_scale.numel() < N or q_min.numel() < N:
+        raise RuntimeError("packed data / scale / min are too short for shape %s" % (tuple(input_shape),))
+    if q_scale.dtype != q_min.dtype:
+        raise RuntimeError("expected scalar type of min to match scale")
+    out = torch.empty(tuple(input_shape), dtype=q_scale.dtype, device=q_input.device)
+    with torch.cuda.device(q_input.device):
+        _abi.check(_abi.lib().gact_dequantize(q_input.data_ptr(), q_bit, q_scale.data_ptr(), q_min.data_ptr(),
+                                              _abi.dtype_code(q_scale.dtype), num_features, out.data_ptr(),
+                                              _abi.stream_of(q_input)))
+    return out

@@ -1,0 +1,126 @@
+/*
+ * C ABI of libgact_hip.so: GACT's saved-activation compression path on MI355X (gfx950).
+ *
+ * Every entry point takes plain device pointers and sizes, launches on the HIP stream it
+ * is given (0 = the null stream), allocates no device memory and returns 0 or a negative
+ * GACT_E* code (gact_strerror() names it).  The current HIP device must be the one the
+ * pointers live on.  Calls are asynchronous; nothing synchronises the stream.
+ *
+ * "Reference" below is LiuXiaoxuanPKU/GACT-ICML; paths are relative to its root.
+ */
+#ifndef GACT_HIP_H
+#define GACT_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GACT_ABI_VERSION 1
+
+/* element types of activations, min, max and scale */
+#define GACT_F32 0
+#define GACT_F16 1
+
+/* where the stochastic-rounding uniform u of each element comes from */
+#define GACT_NOISE_CONST 0  /* u = 0.5: deterministic round-to-nearest                          */
+#define GACT_NOISE_INJECT 1 /* u read from a float tensor laid out like the (padded) data        */
+#define GACT_NOISE_REF 2    /* the reference's stream: one Philox4x32-10 state per output byte,  */
+                            /* (seed, subsequence = byte index, offset 0), cuRAND uniform map    */
+#define GACT_NOISE_FAST 3   /* one Philox4x32-10 block per 8 consecutive elements, 16-bit noise  */
+
+#define GACT_OK 0
+#define GACT_EINVAL (-1) /* bad argument (bits not in {1,2,4,8}, negative size, null pointer ...) */
+#define GACT_EALIGN (-2) /* a pointer is not aligned as the kernels need (16 bytes)               */
+#define GACT_ESHAPE (-3) /* shape not supported by this entry point                               */
+#define GACT_ELAUNCH (-4) /* the HIP runtime reported an error at launch                          */
+#define GACT_EBUDGET (-5) /* calc_precision: every tensor is at 1 bit and the budget is not met   */
+
+const char* gact_strerror(int code);
+int gact_abi_version(void);
+
+/* Bytes the pack kernels write for N groups rows of G*D elements: bits*N_round*G*D/8 with N rounded
+ * up to a multiple of 8/bits.  The reference allocates one byte more and never writes it
+ * (gact/gact/cpp_extension/quantization_cuda_kernel.cu:88-91). */
+int64_t gact_packed_bytes(int bits, int64_t N, int64_t G, int64_t D);
+
+/* Per-row minimum and maximum of a contiguous [N, D] tensor; D % 32 == 0 and D > 32.
+ * Replaces minimax_cuda (gact/gact/cpp_extension/minimax_cuda_kernel.cu:70-89, bound at
+ * minimax.cc:7-14). */
+int gact_minimax(const void* data, int dtype, int64_t N, int64_t D, void* mn, void* mx, void* stream);
+
+/* scale = T(2^bits-1)/(max-min+2e-6) for N*G entries, then the packed codes of data[N,G,D].
+ * Writes gact_packed_bytes() bytes to `packed` and N*G values to `scale`.
+ * Replaces pack_single_precision_cuda (quantization_cuda_kernel.cu:74-146, bound at
+ * quantization.cc:51-61).  `noise` is only read in GACT_NOISE_INJECT mode. */
+int gact_pack(const void* data, const void* mn, const void* mx, int dtype, int bits, int64_t N, int64_t G,
+              int64_t D, int noise_mode, uint64_t seed, const float* noise, void* packed, void* scale,
+              void* stream);
+
+/* out[N,G,D] = T(code)/scale + min.  Replaces unpack_single_precision_cuda
+ * (quantization_cuda_kernel.cu:180-221, bound at quantization.cc:36-49). */
+int gact_unpack(const void* packed, int bits, const void* scale, const void* mn, int dtype, int64_t N,
+                int64_t G, int64_t D, void* out, void* stream);
+
+/* The whole of no_scheme_quantize_pack (gact/gact/ops.py:11-32) for group size 256 in one pass over
+ * the data: `x` holds `numel` contiguous elements, treated as zero-padded to N = ceil(numel/256)
+ * groups; writes min[N], scale[N] (and max[N] when `mx` is not null) and gact_packed_bytes(bits,N,1,256)
+ * bytes.  Same results as gact_minimax + gact_pack on the padded tensor. */
+int gact_quantize(const void* x, int dtype, int64_t numel, int bits, int noise_mode, uint64_t seed,
+                  const float* noise, void* packed, void* scale, void* mn, void* mx, void* stream);
+
+/* The whole of dequantize_and_unpack + the slice of op_dequantize (gact/gact/ops.py:34-47,61-69) for
+ * group size 256: writes exactly `numel` elements. */
+int gact_dequantize(const void* packed, int bits, const void* scale, const void* mn, int dtype,
+                    int64_t numel, void* out, void* stream);
+
+/* Dropout-mask bit packing: n bytes (nonzero = 1) <-> ceil(n/32) int32 words.
+ * Replace act_quantize_dropout_mask_cuda / act_dequantize_dropout_mask_cuda
+ * (quantization_cuda_kernel.cu:254-303, bound at quantization.cc:26-33). */
+int gact_mask_pack(const uint8_t* data, int64_t n, int32_t* mask, void* stream);
+int gact_mask_unpack(const int32_t* mask, int64_t n, uint8_t* out, void* stream);
+
+/* Greedy bit allocation on host memory; mutates b.  Replaces calc_precision
+ * (gact/gact/cpp_extension/calc_precision.cc:66-118, bound at :120-123). */
+int gact_calc_precision(int32_t* b, const float* C, const int64_t* w, int64_t L, double target);
+
+/* The same allocation computed on the GPU from device arrays (b is updated in place), so that the
+ * sensitivities never leave the device.  `status` (device int32, may be null) receives 0 or GACT_EBUDGET.
+ * No counterpart in the reference, which runs calc_precision on the host. */
+int gact_calc_precision_device(int32_t* b, const float* C, const int64_t* w, int64_t L, double target,
+                               int32_t* status, void* stream);
+
+/* One saved tensor of a batched launch.  The table itself lives in device memory. */
+typedef struct gact_batch_entry {
+  const void* x;      /* activation (quantize input / dequantize output), numel elements          */
+  int64_t numel;
+  int32_t dtype;      /* GACT_F32 / GACT_F16                                                       */
+  int32_t reserved;
+  uint64_t seed;      /* per-tensor seed: seeds[tid] + seed_iter (gact/gact/quantizer.py:119-124)  */
+  int64_t first_block; /* exclusive prefix sum of ceil(N/128) over the table (128 groups per block) */
+  int64_t packed_offset; /* byte offset of this tensor's codes in the packed arena (written by     */
+                         /* gact_batch_plan from the device-resident bits)                          */
+  int64_t stats_offset;  /* element offset of this tensor's scale/min rows in the stats arenas      */
+} gact_batch_entry;
+
+/* Fill packed_offset (256-byte aligned, in table order) from device-resident bits; `total` (device
+ * int64, may be null) receives the arena bytes in use.  No counterpart in the reference. */
+int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t* total, void* stream);
+
+/* Quantize / dequantize all L tensors of the table in one grid of `total_blocks` blocks, each tensor at
+ * its own bits[i] in {1,2,4,8} read from device memory.  Scale and min of tensor i are written at
+ * stats_offset (in elements of the tensor's dtype, but the arenas are byte-addressed at 4 bytes per
+ * group so both dtypes share them).  Results equal a loop of gact_quantize / gact_dequantize over the
+ * tensors (gact/gact/quantizer.py:95-142 drives the reference one tensor at a time). */
+int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
+                          int noise_mode, void* packed_arena, void* scale_arena, void* min_arena,
+                          void* stream);
+int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L,
+                            int64_t total_blocks, const void* packed_arena, const void* scale_arena,
+                            const void* min_arena, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GACT_HIP_H */

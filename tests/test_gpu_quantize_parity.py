@@ -1,0 +1,186 @@
+"""HIP kernels against the CPU oracle on the same seeded inputs, through the C ABI.
+
+Bars: packed bytes, scale and the bit allocation bit-exact; min equal by value; dequantized values
+bit-exact (the stated tolerance is 1 ulp; the kernels use an IEEE division, so 0 ulp is asserted).
+The reference's trailing, never-written packed byte is excluded from every comparison.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gact import ops
+from gact.conf import config
+from gact.cpp_extension import _abi
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.float16]
+BITS = [1, 2, 4, 8]
+MODES = {"deterministic": oracle.NOISE_CONST, "reference": oracle.NOISE_REF, "fast": oracle.NOISE_FAST}
+
+
+def make_input(kind, shape, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    if kind == "randn":
+        x = torch.randn(shape, generator=g)
+    elif kind == "relu":
+        x = torch.relu(torch.randn(shape, generator=g))
+    elif kind == "uniform":
+        x = torch.rand(shape, generator=g)
+    elif kind == "wide":
+        x = torch.randn(shape, generator=g) * 100.0
+    else:
+        raise ValueError(kind)
+    return x.to(dtype)
+
+
+def check_quantize(x_cpu, bits, mode_name, seed, noise=None):
+    x = x_cpu.cuda()
+    if noise is not None:
+        q = ops.op_quantize(x, bits, seed, noise=noise.cuda())
+        ref = oracle.op_quantize(x_cpu.numpy(), bits, oracle.NOISE_INJECT, seed, noise.numpy())
+    else:
+        q = ops.op_quantize(x, bits, seed, rng_stream=mode_name)
+        ref = oracle.op_quantize(x_cpu.numpy(), bits, MODES[mode_name], seed)
+    torch.cuda.synchronize()
+    pk, b, sc, mn = q
+    assert b == bits
+    n_written = ref[0].size
+    assert pk.dtype == torch.int8 and pk.numel() == n_written + 1
+    assert sc.shape == ref[2].shape and mn.shape == ref[3].shape
+    got_mn = mn.cpu().numpy()
+    got_sc = sc.cpu().numpy()
+    np.testing.assert_array_equal(got_mn, ref[3])  # by value (+0 == -0)
+    np.testing.assert_array_equal(got_sc.view(np.uint16 if got_sc.dtype == np.float16 else np.uint32),
+                                  ref[2].view(np.uint16 if got_sc.dtype == np.float16 else np.uint32))
+    got_pk = pk.cpu().numpy().view(np.uint8)[:n_written]
+    bad = np.nonzero(got_pk != ref[0])[0]
+    assert bad.size == 0, "packed bytes differ at %d of %d positions, first %s: got %s want %s" % (
+        bad.size, n_written, bad[:5], got_pk[bad[:5]], ref[0][bad[:5]])
+    return q, ref
+
+
+def check_dequantize(q, ref, shape):
+    out = ops.op_dequantize(q, shape)
+    torch.cuda.synchronize()
+    want = oracle.op_dequantize(ref, shape)
+    got = out.cpu().numpy()
+    assert got.shape == tuple(shape) and got.dtype == want.dtype
+    it = np.uint16 if got.dtype == np.float16 else np.uint32
+    bad = np.nonzero(got.view(it).ravel() != want.view(it).ravel())[0]
+    assert bad.size == 0, "dequantized values differ at %d positions, first %s: got %s want %s" % (
+        bad.size, bad[:5], got.ravel()[bad[:5]], want.ravel()[bad[:5]])
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f16"])
+@pytest.mark.parametrize("bits", BITS)
+@pytest.mark.parametrize("mode", list(MODES))
+def test_quantize_dequantize_matches_oracle(dtype, bits, mode):
+    # 1100 groups: not a multiple of 8 groups per row nor of 128 per block, N % wpt != 0 for bits 1
+    shape = (1100, 256) if bits != 1 else (1099, 256)
+    x = make_input("randn", shape, dtype, seed=bits)
+    q, ref = check_quantize(x, bits, mode, seed=42)
+    check_dequantize(q, ref, shape)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f16"])
+@pytest.mark.parametrize("bits", BITS)
+def test_injected_noise_matches_oracle(dtype, bits):
+    shape = (515, 256)
+    x = make_input("relu", shape, dtype, seed=10 + bits)
+    g = torch.Generator().manual_seed(99)
+    noise = torch.rand(shape, generator=g)
+    noise[0, :8] = torch.tensor([0.0, 1.0, 0.5, 0.25, 0.75, 1e-7, 0.9999999, 0.5])
+    q, ref = check_quantize(x, bits, None, seed=0, noise=noise)
+    check_dequantize(q, ref, shape)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f16"])
+@pytest.mark.parametrize("bits", BITS)
+@pytest.mark.parametrize("shape", [(100, 77), (1, 1), (3, 5, 7), (257,), (2, 3, 4, 129), (169343 // 97, 256)])
+def test_ragged_shapes(dtype, bits, shape):
+    # numel not a multiple of 256 (zero-padded last group), N % (8/bits) != 0 (partial last byte fields)
+    x = make_input("relu", shape, dtype, seed=5)
+    q, ref = check_quantize(x, bits, "fast", seed=7)
+    check_dequantize(q, ref, shape)
+    q, ref = check_quantize(x, bits, "deterministic", seed=7)
+    check_dequantize(q, ref, shape)
+
+
+@pytest.mark.parametrize("kind", ["uniform", "wide"])
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f16"])
+@pytest.mark.parametrize("bits", BITS)
+def test_other_distributions(kind, dtype, bits):
+    shape = (640, 256)
+    x = make_input(kind, shape, dtype, seed=3)
+    for mode in ("deterministic", "fast"):
+        q, ref = check_quantize(x, bits, mode, seed=123456)
+        check_dequantize(q, ref, shape)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f16"])
+@pytest.mark.parametrize("bits", BITS)
+def test_edge_groups(dtype, bits):
+    # constant groups (range 0), tiny ranges (half scale overflows to inf), NaN elements, huge values
+    x = torch.zeros((64, 256), dtype=torch.float32)
+    x[0] = 3.0
+    x[1] = -7.5
+    x[2] = torch.linspace(1.0, 1.0 + 1e-4, 256)
+    x[3] = torch.linspace(-1e-6, 1e-6, 256)
+    x[4] = torch.randn(256)
+    x[4, 17] = float("nan")
+    x[5] = torch.randn(256) * 3e4
+    x[6, 0] = 1.0
+    x[7] = torch.rand(256) * 6e-5      # subnormal halves
+    x[8:] = torch.randn(56, 256)
+    x = x.to(dtype)
+    for mode in ("deterministic", "reference", "fast"):
+        q, ref = check_quantize(x, bits, mode, seed=1)
+        out = ops.op_dequantize(q, x.shape).cpu().numpy()
+        want = oracle.op_dequantize(ref, x.shape)
+        np.testing.assert_array_equal(np.isnan(out), np.isnan(want))
+        m = ~np.isnan(want)
+        np.testing.assert_array_equal(out[m], want[m])
+
+
+def test_config1_full_size_deterministic():
+    # BASELINE config 1: fp32 [4096,1024] ~ N(0,1), seed 0, 2 bit, deterministic rounding
+    torch.manual_seed(0)
+    x = torch.randn(4096, 1024)
+    q, ref = check_quantize(x, 2, "deterministic", seed=0)
+    check_dequantize(q, ref, x.shape)
+
+
+def test_one_hot_round_trips_at_one_bit():
+    # tests/test_act_quantized_ops.py:23-38 of the reference: 0/1 data survives 1-bit quantisation exactly
+    config.rng_stream = "fast"
+    for inp in (torch.nn.functional.one_hot(torch.arange(1000), 1000),
+                torch.nn.functional.one_hot(torch.arange(0, 100) % 77)):
+        x = inp.to(torch.float32).cuda()
+        for seed in (0, 1, 2):
+            d = ops.op_dequantize(ops.op_quantize(x, 1, seed), x.shape)
+            assert torch.equal(d.to(torch.uint8), inp.to(torch.uint8).cuda())
+            for stream in ("reference", "deterministic"):
+                d = ops.op_dequantize(ops.op_quantize(x, 1, seed, rng_stream=stream), x.shape)
+                assert torch.equal(d.to(torch.uint8), inp.to(torch.uint8).cuda())
+
+
+def test_big_min_matches_torch_min():
+    # tests/test_act_quantized_ops.py:62-70: (655350, 256) at 4 bit, q_min == torch.min(dim=1)
+    x = torch.rand((65535 * 10, 256), device="cuda")
+    q_input, q_bit, q_scale, q_min = ops.op_quantize(x, 4, 0)
+    assert torch.equal(q_min.reshape(-1), torch.min(x, dim=1).values)
+    rng = torch.max(x, dim=1).values - torch.min(x, dim=1).values  # a float subtraction, then double
+    ref_scale = (15.0 / (rng.double() + 2e-6)).float()
+    assert torch.equal(q_scale.reshape(-1), ref_scale)
+
+
+def test_32bit_passthrough():
+    # tests/test_act_quantized_ops.py:73-91
+    x = torch.rand((2048, 256), device="cuda")
+    q = ops.op_quantize(x, 32, 0)
+    q_input, q_bit, q_scale, q_min = q
+    assert torch.equal(q_min.reshape(-1), torch.min(x, dim=1).values)
+    assert torch.equal(q_scale.reshape(-1), torch.max(x, dim=1).values - torch.min(x, dim=1).values)
+    assert torch.equal(ops.op_dequantize(q, x.shape), x)
