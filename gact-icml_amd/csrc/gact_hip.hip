@@ -659,18 +659,21 @@ calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, cons
 // Batched launch over a table of tensors with device-resident bits.
 // ------------------------------------------------------------------------------------------------
 __global__ void batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int L,
-                                  int64_t* total) {
+                                  int64_t capacity, int64_t* plan) {
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
   int64_t off = 0;
+  bool ok = true;
   for (int t = 0; t < L; t++) {
-    const int bt = bits[t];
-    const int wpt = 8 / (bt > 0 && bt <= 8 ? bt : 8);
+    int bt = bits[t];
+    if (!(bt == 1 || bt == 2 || bt == 4 || bt == 8)) { ok = false; bt = 8; }
+    const int wpt = 8 / bt;
     const int64_t N = (table[t].numel + GROUP - 1) / GROUP;
     const int64_t n_round = (N + wpt - 1) / wpt * wpt;
     table[t].packed_offset = off;
     off += ((int64_t)bt * n_round * (GROUP / 8) + 255) / 256 * 256;
   }
-  if (total) *total = off;
+  plan[0] = off;
+  plan[1] = (ok && off <= capacity) ? 1 : 0;
 }
 
 __device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ table, int L, int64_t block) {
@@ -685,8 +688,9 @@ __device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ t
 template <int NOISE>
 __global__ void __launch_bounds__(256)
 quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
-                        uint8_t* __restrict__ packed_arena, uint8_t* __restrict__ scale_arena,
+                        const int64_t* __restrict__ plan, uint8_t* __restrict__ packed_arena, uint8_t* __restrict__ scale_arena,
                         uint8_t* __restrict__ min_arena) {
+  if (plan[1] == 0) return;  // the plan did not fit the arena or held an invalid width
   const int t = batch_find(table, L, blockIdx.x);
   const gact_batch_entry ent = table[t];
   const int bt = bits[t];
@@ -719,8 +723,9 @@ quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_
 
 __global__ void __launch_bounds__(256)
 dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
-                          const uint8_t* __restrict__ packed_arena, const uint8_t* __restrict__ scale_arena,
+                          const int64_t* __restrict__ plan, const uint8_t* __restrict__ packed_arena, const uint8_t* __restrict__ scale_arena,
                           const uint8_t* __restrict__ min_arena) {
+  if (plan[1] == 0) return;  // the plan did not fit the arena or held an invalid width
   const int t = batch_find(table, L, blockIdx.x);
   const gact_batch_entry ent = table[t];
   const int bt = bits[t];
@@ -1033,46 +1038,49 @@ int gact_calc_precision_device(int32_t* b, const float* C, const int64_t* w, int
   return launch_status();
 }
 
-int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t* total, void* stream) {
-  if (L < 0 || L > (1 << 30)) return GACT_EINVAL;
-  if (L == 0) return GACT_OK;
-  if (!table || !bits) return GACT_EINVAL;
-  hipLaunchKernelGGL(batch_plan_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, table, bits, (int)L, total);
+int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t capacity, int64_t* plan,
+                    void* stream) {
+  if (L < 0 || L > (1 << 30) || capacity < 0) return GACT_EINVAL;
+  if (!plan) return GACT_EINVAL;
+  if (L > 0 && (!table || !bits)) return GACT_EINVAL;
+  hipLaunchKernelGGL(batch_plan_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, table, bits, (int)L, capacity, plan);
   return launch_status();
 }
 
 int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
-                          int noise_mode, void* packed_arena, void* scale_arena, void* min_arena, void* stream) {
+                          int noise_mode, const int64_t* plan, void* packed_arena, void* scale_arena, void* min_arena,
+                          void* stream) {
   if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x7fffffffLL) return GACT_EINVAL;
+  if (noise_mode != GACT_NOISE_CONST && noise_mode != GACT_NOISE_REF && noise_mode != GACT_NOISE_FAST)
+    return GACT_EINVAL;  // injected noise is a single-tensor test mode
   if (L == 0 || total_blocks == 0) return GACT_OK;
-  if (!table || !bits || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
+  if (!table || !bits || !plan || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena)) return GACT_EALIGN;
   const dim3 grid((unsigned)total_blocks), block(256);
   hipStream_t s = (hipStream_t)stream;
   switch (noise_mode) {
     case GACT_NOISE_CONST:
-      hipLaunchKernelGGL((quantize_batched_kernel<GACT_NOISE_CONST>), grid, block, 0, s, table, bits, (int)L, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena);
+      hipLaunchKernelGGL((quantize_batched_kernel<GACT_NOISE_CONST>), grid, block, 0, s, table, bits, (int)L, plan, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena);
       break;
     case GACT_NOISE_REF:
-      hipLaunchKernelGGL((quantize_batched_kernel<GACT_NOISE_REF>), grid, block, 0, s, table, bits, (int)L, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena);
-      break;
-    case GACT_NOISE_FAST:
-      hipLaunchKernelGGL((quantize_batched_kernel<GACT_NOISE_FAST>), grid, block, 0, s, table, bits, (int)L, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena);
+      hipLaunchKernelGGL((quantize_batched_kernel<GACT_NOISE_REF>), grid, block, 0, s, table, bits, (int)L, plan, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena);
       break;
     default:
-      return GACT_EINVAL;  // injected noise is a single-tensor test mode
+      hipLaunchKernelGGL((quantize_batched_kernel<GACT_NOISE_FAST>), grid, block, 0, s, table, bits, (int)L, plan, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena);
+      break;
   }
   return launch_status();
 }
 
 int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
-                            const void* packed_arena, const void* scale_arena, const void* min_arena, void* stream) {
+                            const int64_t* plan, const void* packed_arena, const void* scale_arena,
+                            const void* min_arena, void* stream) {
   if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x7fffffffLL) return GACT_EINVAL;
   if (L == 0 || total_blocks == 0) return GACT_OK;
-  if (!table || !bits || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
+  if (!table || !bits || !plan || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena)) return GACT_EALIGN;
   hipLaunchKernelGGL(dequantize_batched_kernel, dim3((unsigned)total_blocks), dim3(256), 0, (hipStream_t)stream, table, bits, (int)L,
-                     (const uint8_t*)packed_arena, (const uint8_t*)scale_arena, (const uint8_t*)min_arena);
+                     plan, (const uint8_t*)packed_arena, (const uint8_t*)scale_arena, (const uint8_t*)min_arena);
   return launch_status();
 }
 

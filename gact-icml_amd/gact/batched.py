@@ -1,0 +1,151 @@
+"""One launch for many saved tensors of mixed bit widths, with the widths resident on the GPU.
+
+The reference quantizes one tensor per call (gact/gact/quantizer.py:95-142) and computes the widths on
+the host (gact/gact/autoprec.py:188-209).  Here ``calc_precision_device`` leaves the widths in device
+memory, a one-thread planning kernel turns them into packed-arena offsets, and a single grid then
+quantizes (or dequantizes) every tensor at its own width.  Nothing is read back to the host; the
+results are identical to calling ``op_quantize`` / ``op_dequantize`` tensor by tensor.
+
+Grid layout: a block owns 128 groups of 256 elements whatever the width, so the grid
+(sum over tensors of ceil(N_i/128) blocks) is known on the host without knowing the widths.
+"""
+import ctypes
+
+import torch
+
+from .cpp_extension import _abi
+
+GROUPS_PER_BLOCK = 128
+
+
+class BatchedPacked:
+    """What a batched quantize leaves behind: the arenas, the table and the per-tensor geometry."""
+
+    def __init__(self, owner, packed, scale, mn, table, bits, plan, shapes, dtypes, seeds):
+        self.owner = owner
+        self.seeds = list(seeds)
+        self.packed, self.scale, self.min = packed, scale, mn
+        self.table, self.bits, self.plan = table, bits, plan
+        self.shapes, self.dtypes = shapes, dtypes
+
+    def ok(self):
+        """Synchronising check that the plan fitted the arena and every width was valid."""
+        need, ok = self.plan.tolist()
+        return bool(ok), need
+
+    def per_tensor(self, i):
+        """Views (packed bytes, bits, scale[N,1,1], min[N,1,1]) of tensor i in op_quantize's format.
+        Reads the width and the offset back from the device (synchronises)."""
+        b = int(self.bits[i].item())
+        numel = self.owner.numels[i]
+        N = (numel + _abi.GROUP - 1) // _abi.GROUP
+        nbytes = _abi.lib().gact_packed_bytes(b, N, 1, _abi.GROUP)
+        table_host = self.table.cpu().numpy().view("int64").reshape(-1, 7)
+        off = int(table_host[i, 5])
+        so = self.owner.stats_offsets[i] * 4
+        dt = self.dtypes[i]
+        esz = 4 if dt == torch.float32 else 2
+        sc = self.scale[so:so + N * esz].view(dt).reshape(N, 1, 1)
+        mn = self.min[so:so + N * esz].view(dt).reshape(N, 1, 1)
+        return self.packed[off:off + nbytes].view(torch.int8), b, sc, mn
+
+
+class BatchedQuantizer:
+    """Geometry of a fixed list of saved tensors (element counts and dtypes), reusable every iteration."""
+
+    def __init__(self, numels, dtypes, device):
+        if len(numels) != len(dtypes):
+            raise ValueError("one dtype per tensor")
+        self.device = torch.device(device)
+        self.numels = [int(n) for n in numels]
+        self.dtypes = list(dtypes)
+        self.L = len(self.numels)
+        self.first_blocks, self.stats_offsets = [], []
+        blocks = 0
+        groups = 0
+        for n in self.numels:
+            N = (n + _abi.GROUP - 1) // _abi.GROUP
+            self.first_blocks.append(blocks)
+            self.stats_offsets.append(groups)
+            blocks += (N + GROUPS_PER_BLOCK - 1) // GROUPS_PER_BLOCK
+            groups += N
+        self.total_blocks = blocks
+        self.total_groups = groups
+
+    # ---- arena sizing (host-side bounds; the exact need is computed on the device) ----
+    def arena_bytes_for_budget(self, target_bits):
+        """Upper bound of the packed bytes when the widths come from calc_precision with this bit
+        budget: the greedy stops at sum(b_i * numel_i) <= max(target, sum(numel_i)); padding to whole
+        groups, to whole bytes of 8/b groups and to 256-byte offsets adds at most 768 bytes per tensor."""
+        total = max(int(target_bits), sum(self.numels))
+        return (total + 7) // 8 + 768 * self.L + 256
+
+    def arena_bytes_worst_case(self):
+        """Every tensor at 8 bits."""
+        return sum(self.numels) + 768 * self.L + 256
+
+    def _table(self, tensors, seeds):
+        arr = (_abi.BatchEntry * self.L)()
+        for i, t in enumerate(tensors):
+            if t.numel() != self.numels[i] or t.dtype != self.dtypes[i]:
+                raise RuntimeError("tensor %d does not match the geometry this batch was built for" % i)
+            if not t.is_cuda or not t.is_contiguous():
+                raise RuntimeError("tensor %d must be a contiguous CUDA tensor" % i)
+            if not _abi.aligned(t):
+                raise RuntimeError("tensor %d is not 16-byte aligned" % i)
+            e = arr[i]
+            e.x = t.data_ptr()
+            e.numel = self.numels[i]
+            e.dtype = _abi.dtype_code(t.dtype)
+            e.seed = int(seeds[i]) & 0xFFFFFFFFFFFFFFFF
+            e.first_block = self.first_blocks[i]
+            e.packed_offset = 0
+            e.stats_offset = self.stats_offsets[i]
+        host = torch.frombuffer(bytearray(bytes(arr)), dtype=torch.uint8)
+        return host.to(self.device, non_blocking=False)
+
+    def quantize(self, tensors, bits, seeds, arena_bytes=None, rng_stream=None):
+        """Quantize all tensors in one launch.  `bits` is an int32 tensor on the device (e.g. the output
+        of calc_precision_device).  Returns a BatchedPacked; nothing synchronises."""
+        from .cpp_extension.quantization import _noise_mode
+        if bits.dtype != torch.int32 or not bits.is_cuda or bits.numel() != self.L:
+            raise RuntimeError("bits must be an int32 CUDA tensor with one entry per tensor")
+        mode = _noise_mode(None, rng_stream)
+        if arena_bytes is None:
+            arena_bytes = self.arena_bytes_worst_case()
+        lib = _abi.lib()
+        with torch.cuda.device(self.device):
+            table = self._table(tensors, seeds)
+            packed = torch.empty((int(arena_bytes),), dtype=torch.uint8, device=self.device)
+            scale = torch.empty((self.total_groups * 4,), dtype=torch.uint8, device=self.device)
+            mn = torch.empty((self.total_groups * 4,), dtype=torch.uint8, device=self.device)
+            plan = torch.empty((2,), dtype=torch.int64, device=self.device)
+            st = torch.cuda.current_stream(self.device).cuda_stream
+            _abi.check(lib.gact_batch_plan(table.data_ptr(), bits.data_ptr(), self.L, packed.numel(),
+                                           plan.data_ptr(), st))
+            _abi.check(lib.gact_quantize_batched(table.data_ptr(), bits.data_ptr(), self.L, self.total_blocks, mode,
+                                                 plan.data_ptr(), packed.data_ptr(), scale.data_ptr(),
+                                                 mn.data_ptr(), st))
+        # the widths are kept as they were at quantize time: the caller may refresh its own copy
+        return BatchedPacked(self, packed, scale, mn, table, bits.clone(), plan, [t.shape for t in tensors],
+                             list(self.dtypes), seeds)
+
+    def dequantize(self, q, outs=None):
+        """Dequantize every tensor of a BatchedPacked in one launch into fresh tensors (or `outs`)."""
+        lib = _abi.lib()
+        with torch.cuda.device(self.device):
+            if outs is None:
+                outs = [torch.empty(s, dtype=d, device=self.device) for s, d in zip(q.shapes, q.dtypes)]
+            # a fresh table with x pointing at the outputs; planning it again from the same widths gives
+            # the same offsets without reading anything back
+            table = self._table(outs, q.seeds)
+            plan = torch.empty((2,), dtype=torch.int64, device=self.device)
+            st = torch.cuda.current_stream(self.device).cuda_stream
+            _abi.check(lib.gact_batch_plan(table.data_ptr(), q.bits.data_ptr(), self.L, q.packed.numel(),
+                                           plan.data_ptr(), st))
+            _abi.check(lib.gact_dequantize_batched(table.data_ptr(), q.bits.data_ptr(), self.L, self.total_blocks,
+                                                   plan.data_ptr(), q.packed.data_ptr(), q.scale.data_ptr(),
+                                                   q.min.data_ptr(), st))
+            # keep the table alive until the stream has consumed it
+            q._dq_table = (table, plan)
+        return outs

@@ -1,0 +1,170 @@
+"""The extension-style entry points (minimax, pack/unpack_single_precision, dropout masks,
+calc_precision on the device, the batched launch) against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gact import ops
+from gact.batched import BatchedQuantizer
+from gact.cpp_extension import _abi
+from gact.cpp_extension import calc_precision as ext_calc_precision
+from gact.cpp_extension import minimax as ext_minimax
+from gact.cpp_extension import quantization as ext_quantization
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.float16]
+
+
+def bits_view(a):
+    return a.view(np.uint16 if a.dtype == np.float16 else np.uint32)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f16"])
+@pytest.mark.parametrize("shape", [(1000, 256), (37, 64), (5, 1024), (129, 96), (3, 4096)])
+def test_minimax(dtype, shape):
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(shape, generator=g).to(dtype)
+    mn, mx = ext_minimax.minimax(x.cuda())
+    rmn, rmx = oracle.minimax(x.numpy())
+    np.testing.assert_array_equal(mn.cpu().numpy(), rmn)
+    np.testing.assert_array_equal(mx.cpu().numpy(), rmx)
+    # the library routine the reference's own tests compare with (tests/test_act_quantized_ops.py:67-70)
+    assert torch.equal(mn.cpu(), x.min(dim=1).values) and torch.equal(mx.cpu(), x.max(dim=1).values)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f16"])
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("ngd", [(203, 1, 256), (21, 3, 64), (10, 2, 256), (9, 1, 128)])
+@pytest.mark.parametrize("stream", ["deterministic", "reference", "fast"])
+def test_pack_unpack_entry_points(dtype, bits, ngd, stream):
+    N, G, D = ngd
+    g = torch.Generator().manual_seed(bits)
+    x = torch.randn((N, G, D), generator=g).to(dtype)
+    mn_np, mx_np = oracle.minimax(x.reshape(N * G, D).numpy())
+    mode = {"deterministic": 0, "reference": 2, "fast": 3}[stream]
+    sc_np = oracle.scale(mn_np, mx_np, bits)
+    want = oracle.pack(x.numpy(), mn_np, sc_np, bits, mode, 17)
+
+    xd = x.cuda()
+    mn = torch.from_numpy(mn_np).reshape(N, G, 1).cuda()
+    mx = torch.from_numpy(mx_np).reshape(N, G, 1).cuda()
+    packed, scale = ext_quantization.pack_single_precision(xd, mn, mx, bits, True, 17, rng_stream=stream)
+    assert packed.dtype == torch.int8 and packed.numel() == want.size + 1
+    assert scale.shape == (N, G, 1) and scale.dtype == dtype
+    np.testing.assert_array_equal(bits_view(scale.cpu().numpy().reshape(-1)), bits_view(sc_np))
+    np.testing.assert_array_equal(packed.cpu().numpy().view(np.uint8)[:want.size], want)
+
+    out = ext_quantization.unpack_single_precision(packed, bits, scale, mn, N, G, D)
+    assert out.shape == (N, G, D) and out.dtype == dtype
+    ref = oracle.unpack(want, bits, sc_np, mn_np, N, G, D)
+    np.testing.assert_array_equal(bits_view(out.cpu().numpy().reshape(-1)), bits_view(ref.reshape(-1)))
+
+
+def test_pack_uses_the_min_max_it_is_given():
+    # the entry point's contract: codes are taken against the caller's min / max, whatever the data holds
+    x = torch.rand((16, 1, 256)) * 0.5 + 0.25
+    mn = torch.zeros((16, 1, 1))
+    mx = torch.ones((16, 1, 1))
+    packed, scale = ext_quantization.pack_single_precision(x.cuda(), mn.cuda(), mx.cuda(), 4, True, 0,
+                                                           rng_stream="deterministic")
+    sc = oracle.scale(mn.numpy().ravel(), mx.numpy().ravel(), 4)
+    want = oracle.pack(x.numpy(), mn.numpy().ravel(), sc, 4, 0, 0)
+    np.testing.assert_array_equal(packed.cpu().numpy().view(np.uint8)[:want.size], want)
+
+
+@pytest.mark.parametrize("n", [1, 31, 32, 33, 511, 512, 513, 1024, 1000 * 1000, 512 * 7 + 100, 77 * 100])
+def test_dropout_mask(n):
+    g = torch.Generator().manual_seed(n)
+    data = (torch.rand(n, generator=g) < 0.3).to(torch.uint8)
+    q = ops.op_quantize_mask(data.cuda())
+    assert q[0].dtype == torch.int32 and q[0].numel() == (n + 31) // 32
+    np.testing.assert_array_equal(q[0].cpu().numpy(), oracle.mask_pack(data.numpy()))
+    out = ops.op_dequantize_mask(q)
+    assert out.dtype == torch.uint8 and torch.equal(out.cpu(), data)
+
+
+def test_dropout_mask_one_hot_identity():
+    # tests/test_act_quantized_ops.py:16-21 of the reference
+    data = torch.nn.functional.one_hot(torch.arange(1000), 1000).to(torch.uint8).cuda()
+    out = ops.op_dequantize_mask(ops.op_quantize_mask(data))
+    assert out.shape == data.shape and torch.equal(out, data)
+
+
+def _swin_like(rng, L):
+    shapes = [(8, 3136, 96), (8, 784, 192), (8, 196, 384), (8, 49, 768)]
+    return [shapes[rng.integers(0, 4)] for _ in range(L)]
+
+
+@pytest.mark.parametrize("L,init,avg", [(120, 8, 2.0), (120, 32, 2.0), (7, 8, 3.0), (64, 8, 1.0), (65, 8, 4.0),
+                                        (300, 32, 2.5)])
+def test_calc_precision_device_matches_host_and_oracle(L, init, avg):
+    rng = np.random.default_rng(L)
+    C = np.exp(rng.normal(0, 2, L)).astype(np.float32)
+    w = np.array([int(np.prod(s)) for s in _swin_like(rng, L)], dtype=np.int64)
+    target = avg * float(w.sum())
+    want = oracle.calc_precision(np.full(L, init, np.int32), C, w, target)
+    host = ext_calc_precision.calc_precision(torch.full((L,), init, dtype=torch.int32), torch.from_numpy(C),
+                                             torch.from_numpy(w), target)
+    np.testing.assert_array_equal(host.numpy(), want)
+    status = torch.full((1,), 99, dtype=torch.int32, device="cuda")
+    dev = ext_calc_precision.calc_precision_device(torch.full((L,), init, dtype=torch.int32, device="cuda"),
+                                                   torch.from_numpy(C).cuda(), torch.from_numpy(w).cuda(), target,
+                                                   status)
+    np.testing.assert_array_equal(dev.cpu().numpy(), want)
+    assert status.item() == 0
+
+
+def test_calc_precision_device_reports_unreachable_budget():
+    L = 5
+    b = torch.full((L,), 8, dtype=torch.int32, device="cuda")
+    status = torch.zeros((1,), dtype=torch.int32, device="cuda")
+    ext_calc_precision.calc_precision_device(b, torch.ones(L, device="cuda"),
+                                             torch.full((L,), 256, dtype=torch.int64, device="cuda"), 100.0, status)
+    assert status.item() == -5 and b.cpu().tolist() == [1] * L
+
+
+@pytest.mark.parametrize("stream", ["deterministic", "fast", "reference"])
+def test_batched_equals_tensor_by_tensor(stream):
+    rng = np.random.default_rng(3)
+    L = 24
+    shapes = _swin_like(rng, L) + [(100, 77), (3, 5)]
+    dtypes = [torch.float16 if i % 3 else torch.float32 for i in range(len(shapes))]
+    L = len(shapes)
+    g = torch.Generator().manual_seed(0)
+    tensors = [torch.randn(s, generator=g).to(d).cuda() for s, d in zip(shapes, dtypes)]
+    C = np.exp(rng.normal(0, 2, L)).astype(np.float32)
+    w = np.array([t.numel() for t in tensors], dtype=np.int64)
+    target = 2.0 * float(w.sum())
+    bits = ext_calc_precision.calc_precision_device(torch.full((L,), 8, dtype=torch.int32, device="cuda"),
+                                                    torch.from_numpy(C).cuda(), torch.from_numpy(w).cuda(), target)
+    seeds = [i + 5 for i in range(L)]
+    bq = BatchedQuantizer([t.numel() for t in tensors], dtypes, "cuda")
+    q = bq.quantize(tensors, bits, seeds, arena_bytes=bq.arena_bytes_for_budget(target), rng_stream=stream)
+    ok, need = q.ok()
+    assert ok and need <= q.packed.numel()
+    outs = bq.dequantize(q)
+    torch.cuda.synchronize()
+    host_bits = bits.cpu().tolist()
+    assert set(host_bits) <= {1, 2, 4, 8} and len(set(host_bits)) > 1
+    for i, t in enumerate(tensors):
+        single = ops.op_quantize(t, host_bits[i], seeds[i], rng_stream=stream)
+        pk, b, sc, mn = q.per_tensor(i)
+        assert b == host_bits[i]
+        n = pk.numel()
+        assert torch.equal(pk, single[0][:n]), "packed bytes of tensor %d differ" % i
+        assert torch.equal(sc.view(torch.int16 if t.dtype == torch.float16 else torch.int32),
+                           single[2].view(torch.int16 if t.dtype == torch.float16 else torch.int32))
+        assert torch.equal(mn, single[3])
+        d = ops.op_dequantize(single, t.shape)
+        assert torch.equal(outs[i], d), "dequantized tensor %d differs" % i
+
+
+def test_batched_refuses_an_arena_that_is_too_small():
+    tensors = [torch.randn(4096, 256, device="cuda") for _ in range(3)]
+    bq = BatchedQuantizer([t.numel() for t in tensors], [torch.float32] * 3, "cuda")
+    bits = torch.full((3,), 8, dtype=torch.int32, device="cuda")
+    q = bq.quantize(tensors, bits, [0, 1, 2], arena_bytes=1 << 20)
+    ok, need = q.ok()
+    assert not ok and need == 3 * 4096 * 256
