@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Throughput of the saved-activation compression path on one MI355X.
+
+One step = one fused quantize (min/max + scale + stochastic rounding + pack) followed by one
+dequantize (unpack + affine) of one synthetic activation tensor, through the C ABI, with the input
+already resident in HBM.  The default workload is BASELINE.json's configs[1]: a ResNet-50 conv
+activation, fp32 NCHW [128,256,56,56], post-ReLU, group 256, 4 bit, stochastic rounding with Philox
+seed 42.  Bytes are the algorithmic input + output bytes of both directions:
+numel*sizeof(T) + packed bytes + 2*N*sizeof(T) per direction.
+
+Prints ONE JSON line.  `roofline` is for the slower of the two kernels, timed with events on the
+stream the kernels run on inside the timed region; `cpu_baseline` is the C restatement of the
+reference arithmetic (oracle/) run with OpenMP on the host cores over a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "gact-icml_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
+# a copy kernel of known size (see profiles/); None until measured for the workload
+TRAFFIC_BYTES = {}
+
+WORKLOADS = {
+    # name: (shape, dtype, bits, rng_stream, data kind, description)
+    "config1": ((4096, 1024), "float32", 2, "deterministic", "randn",
+                "fp32 [4096,1024] ~N(0,1), 2 bit, deterministic rounding"),
+    "config2": ((128, 256, 56, 56), "float32", 4, "fast", "relu",
+                "ResNet-50 conv activation fp32 [128,256,56,56] post-ReLU, 4 bit, stochastic rounding, Philox seed 42"),
+    "config2-refstream": ((128, 256, 56, 56), "float32", 4, "reference", "relu",
+                          "config2 with the reference's one-Philox-state-per-byte noise stream"),
+    "config3-hidden": ((16384, 1024), "float16", 8, "fast", "randn", "BERT-large hidden states fp16, 8 bit"),
+    "config3-gelu": ((16384, 4096), "float16", 4, "fast", "randn", "BERT-large GELU inputs fp16, 4 bit"),
+    "config3-probs": ((32, 16, 512, 512), "float16", 2, "fast", "softmax", "BERT-large attention probs fp16, 2 bit"),
+    "config4": ((169343, 256), "float32", 1, "fast", "relu60", "GCN node features fp32 [169343,256], ~60% zeros, 1 bit"),
+}
+
+
+def make_input(torch, shape, dtype, kind, seed=0):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    x = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32)
+    if kind == "relu":
+        x = torch.relu(x)
+    elif kind == "relu60":
+        x = torch.relu(x - 0.2533)  # P(N(0,1) < 0.2533) = 0.6
+    elif kind == "softmax":
+        x = torch.softmax(x, dim=-1)
+    return x.to(getattr(torch, dtype)).contiguous()
+
+
+def algorithmic_bytes(numel, esize, bits):
+    N = (numel + 255) // 256
+    wpt = 8 // bits
+    n_round = (N + wpt - 1) // wpt * wpt
+    return numel * esize + n_round * 32 * bits + 2 * N * esize
+
+
+def run_workload(torch, name, steps, warmup, seed=42):
+    from gact.cpp_extension import _abi
+
+    shape, dtype, bits, stream, kind, desc = WORKLOADS[name]
+    lib = _abi.lib()
+    x = make_input(torch, shape, dtype, kind)
+    numel = x.numel()
+    N = (numel + 255) // 256
+    esize = x.element_size()
+    packed = torch.empty((lib.gact_packed_bytes(bits, N, 1, 256) + 1,), dtype=torch.int8, device="cuda")
+    scale = torch.empty((N,), dtype=x.dtype, device="cuda")
+    mn = torch.empty((N,), dtype=x.dtype, device="cuda")
+    out = torch.empty_like(x)
+    st = torch.cuda.current_stream().cuda_stream
+    dt = _abi.dtype_code(x.dtype)
+    mode = _abi.NOISE_MODES[stream]
+
+    def quantize():
+        _abi.check(lib.gact_quantize(x.data_ptr(), dt, numel, bits, mode, seed, None, packed.data_ptr(),
+                                     scale.data_ptr(), mn.data_ptr(), None, st))
+
+    def dequantize():
+        _abi.check(lib.gact_dequantize(packed.data_ptr(), bits, scale.data_ptr(), mn.data_ptr(), dt, numel,
+                                       out.data_ptr(), st))
+
+    for _ in range(warmup):
+        quantize()
+        dequantize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        ev[k][0].record()
+        quantize()
+        ev[k][1].record()
+        dequantize()
+        ev[k][2].record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+
+    per_dir = algorithmic_bytes(numel, esize, bits)
+    q_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / steps
+    d_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / steps
+    wall_ms = (t1 - t0) * 1e3 / steps
+    res = {
+        "workload": name, "desc": desc, "shape": list(shape), "dtype": dtype, "bits": bits, "rng_stream": stream,
+        "bytes_per_direction": per_dir, "ms_per_step": wall_ms,
+        "gbs": 2 * per_dir / (wall_ms * 1e-3) / 1e9,
+        "quantize": {"ms": q_ms, "gbs": per_dir / (q_ms * 1e-3) / 1e9},
+        "dequantize": {"ms": d_ms, "gbs": per_dir / (d_ms * 1e-3) / 1e9},
+    }
+    return res, x
+
+
+def cpu_baseline(torch, x, bits, stream, budget_s=12.0):
+    """The C restatement on the host cores over a leading slice of the same tensor."""
+    import numpy as np
+
+    import oracle
+
+    mode = {"deterministic": oracle.NOISE_CONST, "reference": oracle.NOISE_REF, "fast": oracle.NOISE_FAST}[stream]
+    flat = x.reshape(-1)
+    sample_elems = min(flat.numel(), 256 * 32768)  # 8M elements
+    xs = flat[:sample_elems].cpu().numpy()
+    N = sample_elems // 256
+    groups = xs.reshape(N, 256)
+    esize = xs.dtype.itemsize
+
+    def one_pass():
+        q = oracle.op_quantize(groups, bits, mode, 42)
+        oracle.op_dequantize(q, groups.shape)
+
+    one_pass()  # warm-up (also builds / loads the library)
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        one_pass()
+        reps += 1
+        if time.perf_counter() - t0 >= budget_s:
+            break
+    dt = (time.perf_counter() - t0) / reps
+    per_dir = algorithmic_bytes(sample_elems, esize, bits)
+    return {
+        "value": 2 * per_dir / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
+        "sample": "first %d of %d elements of the same tensor (%d groups), %d quantize+dequantize passes of the C "
+                  "restatement (oracle/gact_oracle.c, OpenMP) in %.1f s" % (sample_elems, flat.numel(), N, reps, dt * reps),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS))
+    ap.add_argument("--all", action="store_true", help="also time the other single-tensor workloads (extra key)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path has no cross-GPU step (each rank compresses its own "
+                 "activations); run with --gpus 1")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    torch.cuda.set_device(0)
+
+    res, x = run_workload(torch, args.workload, args.steps, args.warmup)
+    dom = "quantize" if res["quantize"]["ms"] >= res["dequantize"]["ms"] else "dequantize"
+    achieved = res[dom]["gbs"]
+    line = {
+        "metric": "quantize+dequantize GB/s (algorithmic input+output bytes), 1xMI355X, group=256",
+        "value": res["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if res["dtype"] == "float32" else "f16", "data": "synthetic",
+        "config": {"workload": "%s: %s" % (args.workload, res["desc"]), "bits": res["bits"], "group_size": 256,
+                   "rng_stream": res["rng_stream"], "bytes_per_step": 2 * res["bytes_per_direction"]},
+        "frac_of_hbm_peak": res["gbs"] / HBM_PEAK_GBS,
+        "kernels": {"quantize": res["quantize"], "dequantize": res["dequantize"]},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get((args.workload, dom))},
+    }
+    if args.all:
+        extra = []
+        for name in sorted(WORKLOADS):
+            if name == args.workload:
+                continue
+            r, _ = run_workload(torch, name, max(20, args.steps // 4), max(3, args.warmup // 4))
+            extra.append(r)
+            torch.cuda.empty_cache()
+        line["other_workloads"] = extra
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(torch, x, res["bits"], res["rng_stream"])
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -85,6 +85,28 @@ __device__ __forceinline__ float fast_uniform_map(uint32_t h) {
   return __builtin_fmaf((float)h, 0x1p-16f, 0x1p-17f);
 }
 
+// Activations and codes are touched exactly once per kernel: load and store them with the streaming
+// (nontemporal) hint so that they do not displace each other in L2 / Infinity Cache.
+#ifndef GACT_STREAMING
+#define GACT_STREAMING 1
+#endif
+template <typename V>
+__device__ __forceinline__ V stream_load(const V* p) {
+#if GACT_STREAMING
+  return __builtin_nontemporal_load(p);
+#else
+  return *p;
+#endif
+}
+template <typename V>
+__device__ __forceinline__ void stream_store(V v, V* p) {
+#if GACT_STREAMING
+  __builtin_nontemporal_store(v, p);
+#else
+  *p = v;
+#endif
+}
+
 // ------------------------------------------------------------------------------------------------
 // Per-type pieces.
 // ------------------------------------------------------------------------------------------------
@@ -93,16 +115,23 @@ template <typename T> struct Elem;
 template <> struct Elem<float> {
   static constexpr int kDtype = GACT_F32;
   __device__ static __forceinline__ void load8(const float* p, float (&v)[8]) {
-    f32x4 a = *reinterpret_cast<const f32x4*>(p);
-    f32x4 b = *reinterpret_cast<const f32x4*>(p + 4);
+    f32x4 a = stream_load(reinterpret_cast<const f32x4*>(p));
+    f32x4 b = stream_load(reinterpret_cast<const f32x4*>(p + 4));
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
     v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
   }
   __device__ static __forceinline__ void store8(float* p, const float (&v)[8]) {
     f32x4 a = {v[0], v[1], v[2], v[3]};
     f32x4 b = {v[4], v[5], v[6], v[7]};
-    *reinterpret_cast<f32x4*>(p) = a;
-    *reinterpret_cast<f32x4*>(p + 4) = b;
+    stream_store(a, reinterpret_cast<f32x4*>(p));
+    stream_store(b, reinterpret_cast<f32x4*>(p + 4));
+  }
+  // dequantize layout: 4 chunks of 4 columns, 4i + 64m, so that every store instruction of a row is one
+  // contiguous 256-byte run
+  static constexpr int kDqChunks = 4, kDqWidth = 4;
+  __device__ static __forceinline__ void store_chunk(float* p, const float (&v)[4]) {
+    f32x4 a = {v[0], v[1], v[2], v[3]};
+    stream_store(a, reinterpret_cast<f32x4*>(p));
   }
   __device__ static __forceinline__ float to_float(float v) { return v; }
   __device__ static __forceinline__ float from_float(float v) { return v; }
@@ -129,7 +158,7 @@ template <> struct Elem<float> {
 template <> struct Elem<f16> {
   static constexpr int kDtype = GACT_F16;
   __device__ static __forceinline__ void load8(const f16* p, f16 (&v)[8]) {
-    f16x8 a = *reinterpret_cast<const f16x8*>(p);
+    f16x8 a = stream_load(reinterpret_cast<const f16x8*>(p));
 #pragma unroll
     for (int e = 0; e < 8; e++) v[e] = a[e];
   }
@@ -137,8 +166,11 @@ template <> struct Elem<f16> {
     f16x8 a;
 #pragma unroll
     for (int e = 0; e < 8; e++) a[e] = v[e];
-    *reinterpret_cast<f16x8*>(p) = a;
+    stream_store(a, reinterpret_cast<f16x8*>(p));
   }
+  // dequantize layout: 2 chunks of 8 columns, 8i + 128m (16-byte stores, 256 contiguous bytes per row)
+  static constexpr int kDqChunks = 2, kDqWidth = 8;
+  __device__ static __forceinline__ void store_chunk(f16* p, const f16 (&v)[8]) { store8(p, v); }
   __device__ static __forceinline__ float to_float(f16 v) { return (float)v; }
   __device__ static __forceinline__ f16 from_float(float v) { return (f16)v; }
   __device__ static __forceinline__ float init_lo() { return __builtin_inff(); }  // half(1e30) is +inf
@@ -205,25 +237,20 @@ __device__ __forceinline__ void store_group(T* __restrict__ out, int64_t numel, 
 }
 
 // ------------------------------------------------------------------------------------------------
-// Quantize: the 8 groups of one row.
+// Quantize one super-group: the 8/BITS consecutive groups whose codes share output bytes.
 //   GIVEN = false: min/max are reduced here (fused minimax + scale + pack, one read of x).
 //   GIVEN = true : min/max are read from mn_io / mx_io (the pack entry point's contract).
 // Codes follow quantization_cuda_kernel.cu:38-71; see Elem<T>::code for the arithmetic.
 // ------------------------------------------------------------------------------------------------
 template <typename T, int BITS, int NOISE, bool GIVEN>
-__device__ __forceinline__ void quantize_row(const T* __restrict__ x, int64_t numel, int64_t N, int64_t row,
-                                             int i, uint8_t* __restrict__ packed, T* __restrict__ scale_out,
-                                             T* mn_io, T* mx_io, uint64_t seed,
-                                             const float* __restrict__ noise) {
+__device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int64_t numel, int64_t N, int64_t sg,
+                                                    int i, uint8_t* __restrict__ packed, T* __restrict__ scale_out,
+                                                    T* mn_io, T* mx_io, uint32_t k0, uint32_t k1,
+                                                    const float* __restrict__ noise) {
   constexpr int WPT = 8 / BITS;
   constexpr int QMAX = (1 << BITS) - 1;
-  const uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
-
-#pragma unroll 1
-  for (int it = 0; it < BITS; it++) {  // BITS super-groups of WPT groups = 8 groups
-    const int64_t sg = row * BITS + it;
+  {
     const int64_t n0 = sg * WPT;
-    if (n0 >= N) break;
 
     T v[WPT][2][8];
     T lo_t[WPT], s_t[WPT];
@@ -327,12 +354,75 @@ __device__ __forceinline__ void quantize_row(const T* __restrict__ x, int64_t nu
       u32x2 w;
       w.x = (bytes[k][0] & 0xffu) | ((bytes[k][1] & 0xffu) << 8) | ((bytes[k][2] & 0xffu) << 16) | (bytes[k][3] << 24);
       w.y = (bytes[k][4] & 0xffu) | ((bytes[k][5] & 0xffu) << 8) | ((bytes[k][6] & 0xffu) << 16) | (bytes[k][7] << 24);
-      *reinterpret_cast<u32x2*>(packed + sg * GROUP + chunk_col(k, i)) = w;
+      stream_store(w, reinterpret_cast<u32x2*>(packed + sg * GROUP + chunk_col(k, i)));
     }
   }
 }
 
-// Dequantize: the 8 groups of one row.  quantization_cuda_kernel.cu:149-177.
+// Dequantize one super-group.  quantization_cuda_kernel.cu:149-177.
+template <typename T, int BITS>
+__device__ __forceinline__ void dequantize_supergroup(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
+                                                      const T* __restrict__ mn, int64_t numel, int64_t N, int64_t sg,
+                                                      int i, T* __restrict__ out) {
+  constexpr int WPT = 8 / BITS;
+  constexpr int CH = Elem<T>::kDqChunks, W = Elem<T>::kDqWidth;  // chunk m covers columns W*i + 16*W*m .. +W-1
+  const int64_t n0 = sg * WPT;
+  uint32_t w[CH][W / 4];
+#pragma unroll
+  for (int m = 0; m < CH; m++) {
+    const uint8_t* p = packed + sg * GROUP + W * i + 16 * W * m;
+    if (W == 4) {
+      w[m][0] = stream_load(reinterpret_cast<const uint32_t*>(p));
+    } else {
+      u32x2 t = stream_load(reinterpret_cast<const u32x2*>(p));
+      w[m][0] = t.x;
+      w[m][W / 4 - 1] = t.y;
+    }
+  }
+#pragma unroll
+  for (int ni = 0; ni < WPT; ni++) {
+    const int64_t n = n0 + ni;
+    if (n < N) {
+      const T s = scale[n];
+      const T mv = mn[n];
+      const int64_t base = n * GROUP;
+      const bool full = base + GROUP <= numel;
+#pragma unroll
+      for (int m = 0; m < CH; m++) {
+        T v[W];
+#pragma unroll
+        for (int e = 0; e < W; e++) {
+          int c = (int)__builtin_amdgcn_ubfe(w[m][e >> 2], 8 * (e & 3) + ni * BITS, BITS);
+          v[e] = Elem<T>::decode(c, s, mv);
+        }
+        const int64_t at = base + W * i + 16 * W * m;
+        if (full) {
+          Elem<T>::store_chunk(out + at, v);
+        } else {
+#pragma unroll
+          for (int e = 0; e < W; e++)
+            if (at + e < numel) out[at + e] = v[e];
+        }
+      }
+    }
+  }
+}
+
+// The 8 groups (BITS super-groups) of one row, one after the other: the batched launch, whose grid must
+// not depend on the widths.
+template <typename T, int BITS, int NOISE, bool GIVEN>
+__device__ __forceinline__ void quantize_row(const T* __restrict__ x, int64_t numel, int64_t N, int64_t row, int i,
+                                             uint8_t* __restrict__ packed, T* __restrict__ scale_out, T* mn_io,
+                                             T* mx_io, uint64_t seed, const float* __restrict__ noise) {
+  constexpr int WPT = 8 / BITS;
+#pragma unroll 1
+  for (int it = 0; it < BITS; it++) {
+    const int64_t sg = row * BITS + it;
+    if (sg * WPT >= N) break;
+    quantize_supergroup<T, BITS, NOISE, GIVEN>(x, numel, N, sg, i, packed, scale_out, mn_io, mx_io, (uint32_t)seed,
+                                               (uint32_t)(seed >> 32), noise);
+  }
+}
 template <typename T, int BITS>
 __device__ __forceinline__ void dequantize_row(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
                                                const T* __restrict__ mn, int64_t numel, int64_t N, int64_t row,
@@ -341,29 +431,8 @@ __device__ __forceinline__ void dequantize_row(const uint8_t* __restrict__ packe
 #pragma unroll 1
   for (int it = 0; it < BITS; it++) {
     const int64_t sg = row * BITS + it;
-    const int64_t n0 = sg * WPT;
-    if (n0 >= N) break;
-    u32x2 w[2];
-#pragma unroll
-    for (int k = 0; k < 2; k++) w[k] = *reinterpret_cast<const u32x2*>(packed + sg * GROUP + chunk_col(k, i));
-#pragma unroll
-    for (int ni = 0; ni < WPT; ni++) {
-      const int64_t n = n0 + ni;
-      if (n < N) {
-        const T s = scale[n];
-        const T m = mn[n];
-        T v[2][8];
-#pragma unroll
-        for (int k = 0; k < 2; k++)
-#pragma unroll
-          for (int e = 0; e < 8; e++) {
-            uint32_t word = (e < 4) ? w[k].x : w[k].y;
-            int c = (int)__builtin_amdgcn_ubfe(word, 8 * (e & 3) + ni * BITS, BITS);
-            v[k][e] = Elem<T>::decode(c, s, m);
-          }
-        store_group<T>(out, numel, n, i, v);
-      }
-    }
+    if (sg * WPT >= N) break;
+    dequantize_supergroup<T, BITS>(packed, scale, mn, numel, N, sg, i, out);
   }
 }
 
@@ -398,22 +467,24 @@ __device__ __forceinline__ void minimax_row(const T* __restrict__ x, int64_t N, 
 // ------------------------------------------------------------------------------------------------
 // Single-tensor kernels.
 // ------------------------------------------------------------------------------------------------
+// One super-group per 16-lane row: short waves, many of them.
 template <typename T, int BITS, int NOISE, bool GIVEN>
 __global__ void __launch_bounds__(256)
 quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
                 T* __restrict__ scale_out, T* mn_io, T* mx_io, uint64_t seed, const float* __restrict__ noise) {
-  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
-  if (row * ROW_GROUPS >= N) return;
-  quantize_row<T, BITS, NOISE, GIVEN>(x, numel, N, row, threadIdx.x & 15, packed, scale_out, mn_io, mx_io, seed, noise);
+  const int64_t sg = (int64_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
+  if (sg * (8 / BITS) >= N) return;
+  quantize_supergroup<T, BITS, NOISE, GIVEN>(x, numel, N, sg, threadIdx.x & 15, packed, scale_out, mn_io, mx_io,
+                                             (uint32_t)seed, (uint32_t)(seed >> 32), noise);
 }
 
 template <typename T, int BITS>
 __global__ void __launch_bounds__(256)
 dequantize_kernel(const uint8_t* __restrict__ packed, const T* __restrict__ scale, const T* __restrict__ mn,
                   int64_t numel, int64_t N, T* __restrict__ out) {
-  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
-  if (row * ROW_GROUPS >= N) return;
-  dequantize_row<T, BITS>(packed, scale, mn, numel, N, row, threadIdx.x & 15, out);
+  const int64_t sg = (int64_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
+  if (sg * (8 / BITS) >= N) return;
+  dequantize_supergroup<T, BITS>(packed, scale, mn, numel, N, sg, threadIdx.x & 15, out);
 }
 
 template <typename T>
@@ -764,22 +835,19 @@ inline bool valid_bits(int bits) { return bits == 1 || bits == 2 || bits == 4 ||
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline int launch_status() { return hipGetLastError() == hipSuccess ? GACT_OK : GACT_ELAUNCH; }
 
-// rows of 8 groups; 16 rows per 256-thread block, or 4 rows per 64-thread block when the tensor is
-// too small to give every CU a block otherwise
-inline void row_grid(int64_t N, dim3* grid, dim3* block) {
-  const int64_t rows = (N + ROW_GROUPS - 1) / ROW_GROUPS;
-  int threads = 256;
-  if ((rows + 15) / 16 < 2048) threads = 64;
-  const int rows_per_block = threads / 16;
-  *grid = dim3((unsigned)((rows + rows_per_block - 1) / rows_per_block));
-  *block = dim3(threads);
+// one 16-lane row per unit of work (a super-group for quantize / dequantize, 8 groups for minimax);
+// 16 rows per 256-thread block
+inline void row_grid(int64_t rows, dim3* grid, dim3* block) {
+  *grid = dim3((unsigned)((rows + 15) / 16));
+  *block = dim3(256);
 }
+inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8 / bits); }
 
 template <typename T, int BITS, bool GIVEN>
 int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, T* scale, T* mn, T* mx, int noise_mode,
                     uint64_t seed, const float* noise, hipStream_t stream) {
   dim3 grid, block;
-  row_grid(N, &grid, &block);
+  row_grid(supergroups(N, BITS), &grid, &block);
   switch (noise_mode) {
     case GACT_NOISE_CONST:
       hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_CONST, GIVEN>), grid, block, 0, stream, x, numel, N,
@@ -819,7 +887,7 @@ template <typename T>
 int dispatch_dequantize(int bits, const uint8_t* packed, const T* scale, const T* mn, int64_t numel, int64_t N, T* out,
                         hipStream_t stream) {
   dim3 grid, block;
-  row_grid(N, &grid, &block);
+  row_grid(supergroups(N, bits), &grid, &block);
   switch (bits) {
     case 1: hipLaunchKernelGGL((dequantize_kernel<T, 1>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
     case 2: hipLaunchKernelGGL((dequantize_kernel<T, 2>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
@@ -887,7 +955,7 @@ int gact_minimax(const void* data, int dtype, int64_t N, int64_t D, void* mn, vo
   hipStream_t s = (hipStream_t)stream;
   if (D == GROUP && aligned16(data)) {
     dim3 grid, block;
-    row_grid(N, &grid, &block);
+    row_grid((N + ROW_GROUPS - 1) / ROW_GROUPS, &grid, &block);
     if (dtype == GACT_F32)
       hipLaunchKernelGGL((minimax256_kernel<float>), grid, block, 0, s, (const float*)data, N, (float*)mn, (float*)mx);
     else

@@ -22,8 +22,10 @@ GROUP = 256
 
 def build(force=False):
     """Compile the C restatement (and the reference's calc_precision.cc when the checkout is there)."""
-    if force or not os.path.exists(_LIB_PATH):
-        subprocess.run(["make", "-C", _HERE, "-B" if force else "-s", "all"], check=True)
+    src = os.path.join(_HERE, "gact_oracle.c")
+    stale = not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(src)
+    if force or stale:
+        subprocess.run(["make", "-C", _HERE, "-B", "-s", "all"], check=True)
     return _LIB_PATH
 
 
@@ -73,6 +75,8 @@ def lib():
         L.gact_oracle_calc_precision.restype = i32
         L.gact_oracle_mask_pack.argtypes = [vp, i64, vp]
         L.gact_oracle_mask_unpack.argtypes = [vp, i64, vp]
+        L.gact_oracle_num_threads.restype = i32
+        L.gact_oracle_set_num_threads.argtypes = [i32]
         for name in ("gact_oracle_h2f", "gact_oracle_h2f_sw"):
             getattr(L, name).argtypes = [ctypes.c_uint16]
             getattr(L, name).restype = ctypes.c_float
@@ -81,6 +85,15 @@ def lib():
             getattr(L, name).restype = ctypes.c_uint16
         _lib = L
     return _lib
+
+
+def num_threads():
+    """OpenMP threads the C loops run on."""
+    return int(lib().gact_oracle_num_threads())
+
+
+def set_num_threads(n):
+    lib().gact_oracle_set_num_threads(int(n))
 
 
 def _dt(a):

@@ -483,3 +483,13 @@ void gact_oracle_mask_unpack(const int32_t* mask, int64_t n, uint8_t* out) {
   for (int64_t e = full * 512; e < n; e++)
     out[e] = (uint8_t)(((uint32_t)mask[full * 16 + (e - full * 512) / 32] >> ((e - full * 512) % 32)) & 1u);
 }
+
+/* threads the OpenMP loops above use (reported next to the CPU baseline figure) */
+#ifdef _OPENMP
+#include <omp.h>
+int gact_oracle_num_threads(void) { return omp_get_max_threads(); }
+void gact_oracle_set_num_threads(int n) { if (n > 0) omp_set_num_threads(n); }
+#else
+int gact_oracle_num_threads(void) { return 1; }
+void gact_oracle_set_num_threads(int n) { (void)n; }
+#endif
