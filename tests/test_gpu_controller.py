@@ -1,0 +1,96 @@
+"""The hook layer end to end on the GPU: a small network trained under Controller hooks, as the
+reference's integration tests do (tests/test_controller_auto_precision.py, tests/test_bert.py)."""
+import copy
+
+import pytest
+import torch
+import torch.nn as nn
+
+import gact
+from gact.conf import config
+from gact.controller import Controller
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def restore_config():
+    saved = dict(vars(config))
+    yield
+    vars(config).update(saved)
+
+
+def make_net():
+    torch.manual_seed(0)
+    return nn.Sequential(
+        nn.Conv2d(3, 16, 3, padding=1), nn.BatchNorm2d(16), nn.ReLU(),
+        nn.Conv2d(16, 32, 3, padding=1), nn.ReLU(), nn.Dropout(0.1), nn.AdaptiveAvgPool2d(4),
+        nn.Flatten(), nn.Linear(512, 64), nn.ReLU(), nn.Linear(64, 10)).cuda()
+
+
+def grads_under_hooks(level, x, y, net):
+    gact.set_optimization_level(level)
+    ctl = Controller(net)
+    ctl.install_hook()
+    try:
+        torch.manual_seed(1)
+        loss = nn.functional.cross_entropy(net(x), y)
+        loss.backward()
+    finally:
+        ctl.uninstall_hook()
+    return loss.item(), torch.cat([p.grad.ravel() for p in net.parameters()])
+
+
+def test_gradients_under_compression_approach_the_exact_ones():
+    x = torch.randn(16, 3, 32, 32, device="cuda")
+    y = torch.randint(0, 10, (16,), device="cuda")
+    net = make_net()
+    torch.manual_seed(1)
+    loss0 = nn.functional.cross_entropy(net(x), y)
+    loss0.backward()
+    exact = torch.cat([p.grad.ravel() for p in net.parameters()])
+    errs = {}
+    for level in ("L1.2", "L1", "L1.1"):          # fixed 2, 4, 8 bit
+        n2 = copy.deepcopy(net)
+        n2.zero_grad()
+        loss, g = grads_under_hooks(level, x, y, n2)
+        assert abs(loss - loss0.item()) < 1e-5    # the forward pass is untouched
+        errs[level] = ((g - exact).norm() / exact.norm()).item()
+    assert errs["L1.1"] < 0.02 and errs["L1"] < 0.2
+    assert errs["L1.1"] < errs["L1"] < errs["L1.2"]
+
+
+def train(swap, steps=6):
+    vars(config).update(dict(compress_activation=True, auto_prec=True, bit=4, swap=swap, prefetch=swap,
+                             adapt_interval=4, max_bit=32, log_interval=-1))
+    net = make_net()
+    net.eval()      # no dropout / batch statistics: the run must be reproducible bit for bit
+    opt = torch.optim.SGD(net.parameters(), lr=0.05)
+    ctl = Controller(net)
+    ctl.install_hook()
+    torch.manual_seed(3)
+    data = [(torch.randn(8, 3, 32, 32, device="cuda"), torch.randint(0, 10, (8,), device="cuda")) for _ in range(steps)]
+    losses = []
+    try:
+        for x, y in data:
+            def backprop():
+                net.zero_grad()
+                nn.functional.cross_entropy(net(x), y).backward()
+            opt.zero_grad()
+            loss = nn.functional.cross_entropy(net(x), y)
+            loss.backward()
+            opt.step()
+            losses.append(loss.item())
+            ctl.iterate(backprop)
+    finally:
+        ctl.uninstall_hook()
+    return losses, dict(ctl.quantizer.bits)
+
+
+def test_auto_precision_training_is_identical_with_and_without_swap():
+    # tests/test_controller_auto_precision.py:145 of the reference: the losses agree exactly
+    base, bits = train(swap=False)
+    swapped, bits_s = train(swap=True)
+    assert base == swapped and bits == bits_s
+    assert set(bits.values()) <= {1, 2, 4, 8, 32} and len(bits) >= 4
+    assert all(l == l for l in base)              # no NaN

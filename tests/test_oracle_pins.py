@@ -1,0 +1,387 @@
+"""Pins of the CPU oracle (oracle/gact_oracle.c) that do not restate its formulas:
+
+* IEEE half conversion against numpy,
+* Philox4x32-10 against the Random123 known-answer vectors,
+* min/max against the library routine the reference's own tests use,
+* scale and quantisation codes against exact rational arithmetic (fractions.Fraction) with an
+  independently written correct-rounding routine - a dropped term, a missing rounding or an unfused /
+  fused mix-up changes at least one of the brute-forced cases,
+* code invariants the mathematics fixes (min element -> 0, max element -> 2^b-1, monotone codes),
+* the byte layout on hand-built inputs, sizes from the reference's worked shapes,
+* the reference's own known-answer tests (0/1 data survives 1 bit; closed-form relative error on U[0,1)),
+* stochastic-rounding statistics (unbiased mean, variance f(1-f)) for both Philox streams.
+"""
+import math
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+import oracle
+
+BITS = [1, 2, 4, 8]
+
+
+# ---------------------------------------------------------------------------------------------------
+# exact helpers (independent of the oracle)
+# ---------------------------------------------------------------------------------------------------
+def round_fraction(fr, dtype):
+    """Correctly rounded (nearest, ties to even) conversion of an exact rational to a numpy float type."""
+    if fr == 0:
+        return dtype(0.0)
+    # float(Fraction) is correctly rounded to double; use it only to find the neighbourhood
+    guess = dtype(float(fr))
+    if not np.isfinite(guess):
+        return guess
+    lo = np.nextafter(guess, dtype(-np.inf))
+    hi = np.nextafter(guess, dtype(np.inf))
+    best = None
+    for cand in (lo, guess, hi):
+        if not np.isfinite(cand):
+            continue
+        err = abs(Fraction(float(cand)) - fr)
+        even = (int(np.array(cand).view({2: np.uint16, 4: np.uint32, 8: np.uint64}[np.dtype(dtype).itemsize])) & 1) == 0
+        if best is None or err < best[0] or (err == best[0] and even and not best[2]):
+            best = (err, cand, even)
+    return best[1]
+
+
+def F(x):
+    return Fraction(float(x))
+
+
+def exact_scale(mn, mx, bits, dtype):
+    rng = round_fraction(F(mx) - F(mn), dtype)                       # an operation of the tensor type
+    denom = round_fraction(F(rng) + F(2e-6), np.float64)             # double addition
+    q = round_fraction(Fraction(2 ** bits - 1) / F(denom), np.float64)  # double division
+    q32 = round_fraction(F(q), np.float32)                           # narrowing store
+    return q32 if dtype == np.float32 else round_fraction(F(q32), np.float16)
+
+
+def rne_int(fr):
+    fl = math.floor(fr)
+    rem = fr - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        return fl + 1
+    return fl
+
+
+def exact_code(x, mn, s, u, dtype):
+    if dtype == np.float32:
+        t = round_fraction(F(x) - F(mn), np.float32)
+        y = round_fraction(F(t) * F(s) + F(u), np.float32)           # one rounding: fused multiply-add
+    else:
+        t = round_fraction(F(x) - F(mn), np.float16)
+        p = round_fraction(F(t) * F(s), np.float16)
+        y = round_fraction(F(p) + F(u), np.float32)
+    z = F(y) - Fraction(1, 2)                                         # exact in double
+    z = round_fraction(z, np.float32) if z != 0 else np.float32(0)   # narrowing to float
+    return rne_int(F(z)) if z > 0 else 0
+
+
+# ---------------------------------------------------------------------------------------------------
+def test_half_conversions_match_numpy():
+    L = oracle.lib()
+    allh = np.arange(65536, dtype=np.uint16)
+    want = allh.view(np.float16).astype(np.float32)
+    for fn in (L.gact_oracle_h2f, L.gact_oracle_h2f_sw):
+        got = np.array([fn(int(h)) for h in allh[::7]], dtype=np.float32)
+        w = want[::7]
+        assert np.array_equal(got.view(np.uint32)[~np.isnan(w)], w.view(np.uint32)[~np.isnan(w)])
+    rng = np.random.default_rng(0)
+    xs = np.concatenate([rng.standard_normal(3000).astype(np.float32) * np.float32(s)
+                         for s in (1e-8, 6e-8, 1e-5, 6.1e-5, 1e-3, 1, 100, 6.5e4, 1e6)])
+    # exact ties and the values around the largest finite half
+    xs = np.concatenate([xs, np.array([2049.0, 2051.0, 65504.0, 65519.9, 65520.0, 5.9604645e-8, 2.9802322e-8,
+                                       8.940697e-8, -0.0, 0.0], np.float32)])
+    with np.errstate(over="ignore"):
+        ref = xs.astype(np.float16).view(np.uint16)
+    for fn in (L.gact_oracle_f2h, L.gact_oracle_f2h_sw):
+        got = np.array([fn(float(x)) for x in xs], dtype=np.uint16)
+        assert np.array_equal(got, ref)
+
+
+def test_philox_known_answers():
+    # Random123 kat_vectors for philox4x32-10
+    kat = [
+        ([0, 0, 0, 0], [0, 0], [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]),
+        ([0xffffffff] * 4, [0xffffffff] * 2, [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]),
+        ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0],
+         [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1]),
+    ]
+    for ctr, key, want in kat:
+        assert [int(v) for v in oracle.philox4x32_10(ctr, key)] == want
+
+
+def test_curand_uniform_map_closed_form():
+    assert oracle.curand_uniform(0) == 2.0 ** -33
+    assert oracle.curand_uniform(0xFFFFFFFF) == 1.0          # 2^32-1 converts to 2^32: the map reaches 1
+    assert oracle.curand_uniform(1 << 31) == 0.5             # 0.5 + 2^-33 rounds to 0.5
+    rng = np.random.default_rng(1)
+    for x in rng.integers(0, 1 << 32, 200):
+        xf = round_fraction(Fraction(int(x)), np.float32)
+        want = round_fraction(F(xf) * Fraction(1, 1 << 32) + Fraction(1, 1 << 33), np.float32)
+        assert oracle.curand_uniform(int(x)) == float(want)
+
+
+def test_reference_stream_walks_the_counter_like_curand():
+    # draw ni of byte j = word ni%4 of Philox(key=seed, ctr=(ni/4, 0, j lo, j hi))
+    seed, bits, N = 42, 1, 16
+    u = oracle.noise(oracle.NOISE_REF, seed, bits, N)
+    for (n, d) in [(0, 0), (3, 5), (7, 255), (8, 0), (13, 77)]:
+        j = (n // 8) * 256 + d
+        ni = n % 8
+        blk = oracle.philox4x32_10([ni // 4, 0, j, 0], [seed, 0])
+        assert u[n, 0, d] == np.float32(oracle.curand_uniform(int(blk[ni % 4])))
+    # 64-bit seeds and negative C ints (sign-extended to uint64 by the reference's binding)
+    u2 = oracle.noise(oracle.NOISE_REF, (-3) & 0xFFFFFFFFFFFFFFFF, 2, 4)
+    blk = oracle.philox4x32_10([0, 0, 1, 0], [0xFFFFFFFD, 0xFFFFFFFF])
+    assert u2[2, 0, 1] == np.float32(oracle.curand_uniform(int(blk[2])))
+
+
+def test_fast_stream_definition():
+    seed = 7
+    u = oracle.noise(oracle.NOISE_FAST, seed, 4, 3).reshape(-1)
+    for E in (0, 1, 7, 8, 300, 767):
+        blk = oracle.philox4x32_10([0, 0, E // 8, 0], [seed, 0])
+        w = int(blk[(E % 8) // 2])
+        h = (w >> 16) if (E % 2) else (w & 0xFFFF)
+        assert u[E] == np.float32((h + 0.5) / 65536.0)
+    assert 0.0 < u.min() and u.max() < 1.0
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_minimax_is_numpy_min_max(dtype):
+    rng = np.random.default_rng(2)
+    for shape in [(300, 256), (17, 64), (4, 1024)]:
+        x = rng.standard_normal(shape).astype(dtype)
+        x[0, 3] = 0.0
+        x[0, 4] = -0.0
+        mn, mx = oracle.minimax(x)
+        np.testing.assert_array_equal(mn, x.min(axis=1))
+        np.testing.assert_array_equal(mx, x.max(axis=1))
+    # NaNs are skipped (std::min / std::max keep the accumulator)
+    x = rng.standard_normal((2, 64)).astype(dtype)
+    x[0, 5] = np.nan
+    mn, mx = oracle.minimax(x)
+    np.testing.assert_array_equal(mn, np.nanmin(x, axis=1))
+    np.testing.assert_array_equal(mx, np.nanmax(x, axis=1))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bits", BITS)
+def test_scale_against_exact_rational(dtype, bits):
+    rng = np.random.default_rng(bits)
+    mn = rng.standard_normal(60).astype(dtype)
+    mx = (mn.astype(np.float32) + np.abs(rng.standard_normal(60)).astype(np.float32) *
+          np.float32(10.0) ** rng.integers(-6, 3, 60)).astype(dtype)
+    mx[:3] = mn[:3]                                     # range 0
+    got = oracle.scale(mn, mx, bits)
+    with np.errstate(over="ignore"):
+        for i in range(mn.size):
+            want = exact_scale(mn[i], mx[i], bits, dtype)
+            assert got[i] == want or (np.isinf(got[i]) and np.isinf(want)), (i, mn[i], mx[i], got[i], want)
+    # special cases: range 0 -> (2^b-1)/2e-6; a half range below (2^b-1)/65504 overflows to inf
+    if dtype == np.float32:
+        assert got[0] == np.float32((2 ** bits - 1) / 2e-6)
+    else:
+        assert np.isinf(got[0])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bits", BITS)
+def test_codes_against_exact_rational_brute_force(dtype, bits):
+    rng = np.random.default_rng(100 + bits)
+    N = 8 // bits + 1                                   # one full byte row and a partial one
+    x = (rng.standard_normal((N, 1, 64)) * 3).astype(dtype)
+    u = rng.random((N, 1, 64)).astype(np.float32)
+    u[0, 0, :6] = [0.0, 1.0, 0.5, 0.25, 0.75, 2.0 ** -33]
+    mn, mx = oracle.minimax(x.reshape(N, 64))
+    sc = oracle.scale(mn, mx, bits)
+    packed = oracle.pack(x, mn, sc, bits, oracle.NOISE_INJECT, 0, u)
+    wpt = 8 // bits
+    want = np.zeros(packed.size, np.int64)
+    for n in range(N):
+        for d in range(64):
+            c = exact_code(x[n, 0, d], mn[n], sc[n], u[n, 0, d], dtype)
+            # the accumulator is a uint8_t: an over-range code (half rounding can produce 2^b) spills into
+            # the next field and loses what does not fit
+            want[(n // wpt) * 64 + d] |= (c << ((n % wpt) * bits)) & 0xFF
+    np.testing.assert_array_equal(packed, want)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bits", BITS)
+def test_code_invariants(dtype, bits):
+    rng = np.random.default_rng(7)
+    N = 64
+    x = rng.standard_normal((N, 256)).astype(dtype)
+    qmax = 2 ** bits - 1
+    for mode, uval in ((oracle.NOISE_CONST, None), (oracle.NOISE_INJECT, 0.9), (oracle.NOISE_INJECT, 0.1)):
+        u = None if uval is None else np.full((N, 256), uval, np.float32)
+        pk, _, sc, mn, mx = oracle.op_quantize(x, bits, mode, 0, u)
+        codes = unpack_codes(pk, bits, N)
+        assert codes.min() >= 0 and codes.max() <= qmax
+        if dtype == np.float16 and not (uval is not None and uval < 0.5):
+            # half rounding of (x-min)*scale can reach 2^b-1 + 1/4, which u > 0.75 lifts to the code 2^b;
+            # the uint8 accumulator then truncates it (the reference's behaviour).  Only float32 keeps
+            # the "maximum -> 2^b-1" invariant for every u >= 0.5; for half check u = 0.5 below.
+            if uval is not None:
+                continue
+        rows = np.arange(N)
+        # the group minimum always codes 0: y = u <= 1, y - 0.5 <= 0.5, ties to even -> 0
+        assert (codes[rows, x.argmin(axis=1)] == 0).all()
+        # the group maximum codes 2^b-1 when u >= 0.5
+        if uval is None or uval >= 0.5:
+            assert (codes[rows, x.argmax(axis=1)] == qmax).all()
+        # with one u for the whole group the codes are monotone in x
+        order = np.argsort(x.astype(np.float32), axis=1, kind="stable")
+        sorted_codes = np.take_along_axis(codes, order, axis=1)
+        assert (np.diff(sorted_codes, axis=1) >= 0).all()
+
+
+def unpack_codes(packed, bits, N):
+    wpt = 8 // bits
+    n_round = (N + wpt - 1) // wpt * wpt
+    b = np.asarray(packed, np.uint8).reshape(n_round // wpt, 256)
+    out = np.empty((n_round, 256), np.int64)
+    for ni in range(wpt):
+        out[ni::wpt] = (b >> (ni * bits)) & (2 ** bits - 1)
+    return out[:N]
+
+
+@pytest.mark.parametrize("bits", BITS)
+def test_layout_on_constant_coded_groups(bits):
+    # group ni of a byte row holds only its min and its max, the max at a column set that differs per
+    # group; every byte must then be sum(code_ni << ni*bits)
+    wpt = 8 // bits
+    N = 2 * wpt + (1 if wpt > 1 else 0)                 # two full rows + one partial row
+    qmax = 2 ** bits - 1
+    x = np.zeros((N, 256), np.float32)
+    for n in range(N):
+        x[n, (np.arange(256) // (n + 1)) % 2 == 1] = 1.0 + n
+    pk, _, sc, mn, mx = oracle.op_quantize(x, bits, oracle.NOISE_CONST)
+    n_round = (N + wpt - 1) // wpt * wpt
+    assert pk.size == n_round * 32 * bits == oracle.packed_len(bits, N)
+    want = np.zeros((n_round // wpt, 256), np.int64)
+    for n in range(N):
+        want[n // wpt] |= np.where(x[n] > 0, qmax, 0) << ((n % wpt) * bits)
+    np.testing.assert_array_equal(pk.reshape(-1, 256), want)
+
+
+def test_sizes_of_the_reference_shapes():
+    # b=2, N=5: 8 groups after rounding, 512 bytes written, 513 allocated by the reference
+    assert oracle.packed_len(2, 5) == 512
+    # [100,77] -> 7700 elements -> 31 groups; one-hot 1000x1000 -> 3907 groups (tests/test_act_quantized_ops.py)
+    assert oracle.pad_groups(np.zeros((100, 77), np.float32)).shape == (31, 256)
+    assert oracle.pad_groups(np.zeros((1000, 1000), np.float32)).shape == (3907, 256)
+    # BASELINE configs 1, 2 and 4 (packed bytes)
+    assert oracle.packed_len(2, 16384) == 1048576
+    assert oracle.packed_len(4, 401408) == 51380224
+    assert oracle.packed_len(1, 169343) == 5419008
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bits", BITS)
+def test_unpack_inverts_pack_and_follows_the_formula(dtype, bits):
+    rng = np.random.default_rng(9)
+    N = 19
+    x = rng.standard_normal((N, 256)).astype(dtype)
+    q = oracle.op_quantize(x, bits, oracle.NOISE_FAST, 5)
+    codes = unpack_codes(q[0], bits, N)
+    out = oracle.op_dequantize(q, x.shape)
+    sc, mn = q[2].reshape(N), q[3].reshape(N)
+    for n in (0, 7, 18):
+        for d in (0, 100, 255):
+            quo = round_fraction(Fraction(int(codes[n, d])) / F(sc[n]), np.float32)
+            if dtype == np.float16:
+                quo = round_fraction(F(quo), np.float16)
+            want = round_fraction(F(quo) + F(mn[n]), dtype)
+            assert out[n, d] == want
+    # dequantised values stay within one quantisation step of the input
+    step = (x.max(axis=1).astype(np.float64) - x.min(axis=1).astype(np.float64)) / (2 ** bits - 1)
+    err = np.abs(out.astype(np.float64) - x.astype(np.float64))
+    if dtype == np.float32:
+        assert (err <= step[:, None] * 1.02).all()
+    elif bits < 8:
+        # half arithmetic adds rounding of the same order as a fine step; at 8 bits an over-range code of
+        # the group maximum wraps to 0 (the reference's uint8 truncation), so no bound holds there
+        assert (err <= step[:, None] * 1.2 + 1e-2).all()
+
+
+def test_binary_data_round_trips_at_one_bit():
+    # tests/test_act_quantized_ops.py:23-38 of the reference
+    for inp in (np.eye(1000, dtype=np.float32)[:300], np.eye(77, dtype=np.float32)[np.arange(100) % 77]):
+        for mode in (oracle.NOISE_CONST, oracle.NOISE_REF, oracle.NOISE_FAST):
+            for seed in (0, 1):
+                out = oracle.op_dequantize(oracle.op_quantize(inp, 1, mode, seed), inp.shape)
+                np.testing.assert_array_equal(out.astype(np.uint8), inp.astype(np.uint8))
+
+
+def test_32bit_passthrough():
+    rng = np.random.default_rng(3)
+    x = rng.random((64, 256)).astype(np.float32)
+    q = oracle.op_quantize(x, 32)
+    np.testing.assert_array_equal(q[3].reshape(-1), x.min(axis=1))
+    np.testing.assert_array_equal(q[2].reshape(-1), x.max(axis=1) - x.min(axis=1))
+    np.testing.assert_array_equal(oracle.op_dequantize(q, x.shape), x)
+
+
+@pytest.mark.parametrize("mode", [oracle.NOISE_REF, oracle.NOISE_FAST])
+@pytest.mark.parametrize("bits", BITS)
+def test_relative_error_on_uniform_data_matches_closed_form(mode, bits):
+    # stochastic rounding of U[0,1) data: E[(xhat-x)^2] = step^2/6, E[x^2] = 1/3 -> ratio 0.5/(2^b-1)^2
+    # (the quantity tests/test_act_quantized_ops.py:41-60 prints)
+    rng = np.random.default_rng(11)
+    x = rng.random((2048, 256)).astype(np.float32)
+    out = oracle.op_dequantize(oracle.op_quantize(x, bits, mode, 3), x.shape)
+    ratio = ((out - x).astype(np.float64) ** 2).sum() / (x.astype(np.float64) ** 2).sum()
+    want = 0.5 / (2 ** bits - 1) ** 2
+    assert abs(ratio / want - 1) < 0.03, (ratio, want)
+
+
+@pytest.mark.parametrize("mode", [oracle.NOISE_REF, oracle.NOISE_FAST])
+@pytest.mark.parametrize("bits", BITS)
+def test_stochastic_rounding_statistics(mode, bits):
+    # one group quantised under many seeds: mean error within 1e-3 * range, variance = step^2 * f(1-f)
+    rng = np.random.default_rng(5)
+    x = rng.random((1, 256)).astype(np.float32)
+    x[0, 0], x[0, 1] = 0.0, 1.0
+    qmax = 2 ** bits - 1
+    seeds = 4000
+    acc = np.zeros(256)
+    acc2 = np.zeros(256)
+    tiled = np.repeat(x, seeds, axis=0)                 # the same group at 4000 positions = 4000 noise draws
+    out = oracle.op_dequantize(oracle.op_quantize(tiled, bits, mode, 123), tiled.shape).astype(np.float64)
+    err = out - x.astype(np.float64)
+    acc, acc2 = err.mean(axis=0), err.var(axis=0)
+    rng_x = 1.0
+    assert np.abs(acc).max() < 4 * (1.0 / qmax) * 0.5 / math.sqrt(seeds) + 1e-3 * rng_x
+    assert abs(acc.mean()) < 1e-3 * rng_x
+    f = (x[0].astype(np.float64) * qmax) % 1.0
+    want_var = (1.0 / qmax) ** 2 * f * (1 - f)
+    assert abs(acc2.sum() / want_var.sum() - 1) < 0.05
+
+
+def test_both_streams_are_uniform():
+    for mode in (oracle.NOISE_REF, oracle.NOISE_FAST):
+        u = oracle.noise(mode, 99, 2, 2048).astype(np.float64).reshape(-1)
+        assert abs(u.mean() - 0.5) < 2e-3 and abs(u.var() - 1 / 12) < 2e-3
+        hist, _ = np.histogram(u, bins=16, range=(0, 1))
+        assert hist.min() > 0.9 * u.size / 16
+        # different seeds decorrelate
+        v = oracle.noise(mode, 100, 2, 2048).astype(np.float64).reshape(-1)
+        assert abs(np.corrcoef(u, v)[0, 1]) < 0.01
+
+
+@pytest.mark.parametrize("n", [1, 31, 32, 33, 511, 512, 513, 1024, 512 * 3 + 100])
+def test_mask_layout_and_round_trip(n):
+    rng = np.random.default_rng(n)
+    data = (rng.random(n) < 0.4).astype(np.uint8)
+    mask = oracle.mask_pack(data)
+    assert mask.dtype == np.int32 and mask.size == (n + 31) // 32
+    full = n // 512
+    for e in range(0, full * 512, 37):                  # quantization_cuda_kernel.cu:243: word e%16, bit e/16 of its block
+        blk, r = divmod(e, 512)
+        assert ((int(mask[blk * 16 + r % 16]) >> (r // 16)) & 1) == data[e]
+    np.testing.assert_array_equal(oracle.mask_unpack(mask, n), data)
