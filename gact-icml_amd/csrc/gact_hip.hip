@@ -1,15 +1,19 @@
 // GACT saved-activation compression for MI355X (gfx950): per-group min/max, scale, stochastic
 // rounding, bit packing, and the inverse, as hand-written HIP kernels behind a C ABI.
 //
-// Work decomposition (all kernels): a DPP row of 16 lanes owns 8 consecutive groups of 256 elements.
-// Inside a group lane i of the row owns two runs of 8 consecutive columns, 128k + 8i .. +7 (k = 0,1),
-// so every load instruction of a row covers 256 contiguous bytes, per-group reductions are four
-// row_ror DPP steps that never leave the row, and - because the reference packs the SAME column of
-// 8/bits consecutive groups into one byte - the lane that owns a column owns every code of that byte:
-// packing needs no cross-lane traffic at all.  A wave is 4 rows, a workgroup 1 or 4 waves.
+// Quantize: a DPP row of 16 lanes owns one "super-group", the 8/bits consecutive groups of 256
+// elements whose codes share output bytes.  Inside a group lane i of the row owns two runs of 8
+// consecutive columns, 128k + 8i .. +7 (k = 0,1).  Per-group reductions are four row_ror DPP steps that
+// never leave the row, and - because the reference packs the SAME column of 8/bits consecutive groups
+// into one byte - the lane that owns a column owns every code of that byte: packing needs no
+// cross-lane traffic at all.  8 consecutive elements are also what one Philox block feeds.
+//
+// Dequantize has no reduction, so a whole wave owns a super-group: lane l owns columns 4l .. 4l+3, reads
+// one dword of codes, and every store instruction of the wave writes one group contiguously; scale and
+// min are wave-uniform and come through the scalar cache.
 //
 // Floating-point contract: this file is compiled with -ffp-contract=off, so every operation below is
-// the IEEE operation it spells; the one fused multiply-add of the path is written __builtin_fmaf.
+// the IEEE operation it spells; the fused multiply-adds of the path are written __builtin_fmaf.
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -22,12 +26,14 @@
 
 typedef _Float16 f16;
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define GROUP 256
-#define ROW_GROUPS 8 /* groups owned by one 16-lane row */
+#define ROW_GROUPS 8 /* groups owned by one 16-lane row in the minimax and batched kernels */
 
 // ------------------------------------------------------------------------------------------------
 // DPP row reductions (16 lanes).  Rotating by 8, 4, 2, 1 leaves the row-wide result in every lane.
@@ -55,16 +61,20 @@ __device__ __forceinline__ float row_all_max(float v) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Philox4x32-10.  The key schedule only depends on the seed, so it stays on the scalar unit.
+// Philox4x32-10.  The key schedule only depends on the seed, so it stays on the scalar unit; each
+// round is two 32x32->64 multiplies and two three-input XORs (v_bitop3_b32, truth table 0x96).
 // ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t xor3(uint32_t a, uint32_t b, uint32_t c) {
+  return __builtin_amdgcn_bitop3_b32(a, b, c, 0x96);
+}
 __device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
                                               uint32_t k1, uint32_t (&out)[4]) {
 #pragma unroll
   for (int r = 0; r < 10; r++) {
     uint64_t p0 = (uint64_t)0xD2511F53u * c0;
     uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
-    uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
-    uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    uint32_t n0 = xor3((uint32_t)(p1 >> 32), c1, k0);
+    uint32_t n2 = xor3((uint32_t)(p0 >> 32), c3, k1);
     c1 = (uint32_t)p1;
     c3 = (uint32_t)p0;
     c0 = n0;
@@ -107,140 +117,214 @@ __device__ __forceinline__ void stream_store(V v, V* p) {
 #endif
 }
 
+// round-to-nearest-even integer of z clamped below at 0: rint(max(z, 0)) of the reference's
+// __float2int_rn(fmax(z, 0)).  v_cvt_u32_f32 clamps negative inputs and NaN to 0, so no separate max is
+// needed; above 2^32 it saturates to 0xffffffff where the signed conversion saturates to 0x7fffffff -
+// the two agree in every bit the uint8 accumulator keeps once the code is shifted into its field.
+__device__ __forceinline__ uint32_t rint_clamp0(float z) {
+  float r = __builtin_rintf(z);
+  uint32_t c;
+  asm("v_cvt_u32_f32_e32 %0, %1" : "=v"(c) : "v"(r));
+  return c;
+}
+
+// Correctly rounded c / s from the correctly rounded reciprocal r = RN(1/s) (Markstein): q = RN(c*r),
+// e = c - s*q exactly (one FMA), result RN(q + e*r).  Valid for finite nonzero s with a normal quotient;
+// the callers fall back to the division otherwise.
+__device__ __forceinline__ float div_by_reciprocal(float c, float s, float r) {
+  float q = c * r;
+  float e = __builtin_fmaf(-q, s, c);
+  return __builtin_fmaf(e, r, q);
+}
+// s is a scale the quotient c/s (0 <= c <= 255) can be taken through the reciprocal for: finite, and
+// far enough from the ends of the exponent range that neither 1/s nor c/s is subnormal or overflows
+__device__ __forceinline__ bool reciprocal_safe(float s) {
+  float a = __builtin_fabsf(s);
+  return a > 0x1p-100f && a < 0x1p100f;
+}
+
 // ------------------------------------------------------------------------------------------------
-// Per-type pieces.
+// Per-type pieces.  Store holds the 16 elements of one group a quantize lane owns (2 chunks of 8).
 // ------------------------------------------------------------------------------------------------
 template <typename T> struct Elem;
 
 template <> struct Elem<float> {
-  static constexpr int kDtype = GACT_F32;
+  struct Store { float v[2][8]; };
   __device__ static __forceinline__ void load8(const float* p, float (&v)[8]) {
     f32x4 a = stream_load(reinterpret_cast<const f32x4*>(p));
     f32x4 b = stream_load(reinterpret_cast<const f32x4*>(p + 4));
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
     v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
   }
-  __device__ static __forceinline__ void store8(float* p, const float (&v)[8]) {
-    f32x4 a = {v[0], v[1], v[2], v[3]};
-    f32x4 b = {v[4], v[5], v[6], v[7]};
-    stream_store(a, reinterpret_cast<f32x4*>(p));
-    stream_store(b, reinterpret_cast<f32x4*>(p + 4));
-  }
-  // dequantize layout: 4 chunks of 4 columns, 4i + 64m, so that every store instruction of a row is one
-  // contiguous 256-byte run
-  static constexpr int kDqChunks = 4, kDqWidth = 4;
-  __device__ static __forceinline__ void store_chunk(float* p, const float (&v)[4]) {
-    f32x4 a = {v[0], v[1], v[2], v[3]};
-    stream_store(a, reinterpret_cast<f32x4*>(p));
-  }
-  __device__ static __forceinline__ float to_float(float v) { return v; }
-  __device__ static __forceinline__ float from_float(float v) { return v; }
+  __device__ static __forceinline__ void load_chunk(const float* p, Store& st, int k) { load8(p, st.v[k]); }
+  __device__ static __forceinline__ void set(Store& st, int k, int e, float x) { st.v[k][e] = x; }
   __device__ static __forceinline__ float init_lo() { return 1e30f; }
   __device__ static __forceinline__ float init_hi() { return -1e30f; }
+  __device__ static __forceinline__ float from_float(float v) { return v; }
+  __device__ static __forceinline__ void minmax(const Store& st, float& lo, float& hi) {
+#pragma unroll
+    for (int k = 0; k < 2; k++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        lo = __builtin_fminf(lo, st.v[k][e]);
+        hi = __builtin_fmaxf(hi, st.v[k][e]);
+      }
+  }
   // scale = float( double(float(qmax)) / (double(max - min) + 2e-6) )
   __device__ static __forceinline__ float make_scale(float lo, float hi, int qmax) {
     float range = hi - lo;
     return (float)((double)(float)qmax / ((double)range + 2e-6));
   }
   // code = rint(max(fma(x - mn, s, u) - 0.5, 0))
-  __device__ static __forceinline__ int code(float x, float mn, float s, float u) {
-    float t = x - mn;
+  __device__ static __forceinline__ uint32_t code1(const Store& st, int k, int e, float mn, float s, float u) {
+    float t = st.v[k][e] - mn;
     float y = __builtin_fmaf(t, s, u);
-    float z = __builtin_fmaxf(y - 0.5f, 0.0f);
-    return (int)__builtin_rintf(z);
+    return rint_clamp0(y - 0.5f);
   }
-  __device__ static __forceinline__ float decode(int c, float s, float mn) {
-    float q = (float)c / s;
-    return q + mn;
+  template <bool CONST_NOISE>
+  __device__ static __forceinline__ void codes8(const Store& st, int k, float mn, float s, const float (&u)[8],
+                                                uint32_t (&c)[8]) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) c[e] = code1(st, k, e, mn, s, u[e]);
+  }
+
+  // ---- dequantize: out = float(code) / scale + min ----
+  struct Dq { float s, r, mn; bool fast; };
+  __device__ static __forceinline__ Dq dq_prepare(float s, float mn) {
+    Dq d;
+    d.s = s; d.mn = mn;
+    d.fast = reciprocal_safe(s);
+    d.r = 1.0f / s;
+    return d;
+  }
+  __device__ static __forceinline__ float decode(int c, const Dq& d) {
+    float q = d.fast ? div_by_reciprocal((float)c, d.s, d.r) : (float)c / d.s;
+    return q + d.mn;
+  }
+  static constexpr int kDqWidth = 4;  // columns per dequantize lane: one 16-byte store
+  __device__ static __forceinline__ void store_dq(float* p, const float (&v)[4]) {
+    f32x4 a = {v[0], v[1], v[2], v[3]};
+    stream_store(a, reinterpret_cast<f32x4*>(p));
   }
 };
 
 template <> struct Elem<f16> {
-  static constexpr int kDtype = GACT_F16;
-  __device__ static __forceinline__ void load8(const f16* p, f16 (&v)[8]) {
+  struct Store { f16x2 v[2][4]; };   // pairs, so that subtraction and product run as packed ops
+  __device__ static __forceinline__ void load_chunk(const f16* p, Store& st, int k) {
     f16x8 a = stream_load(reinterpret_cast<const f16x8*>(p));
 #pragma unroll
-    for (int e = 0; e < 8; e++) v[e] = a[e];
+    for (int j = 0; j < 4; j++) st.v[k][j] = f16x2{a[2 * j], a[2 * j + 1]};
   }
-  __device__ static __forceinline__ void store8(f16* p, const f16 (&v)[8]) {
-    f16x8 a;
-#pragma unroll
-    for (int e = 0; e < 8; e++) a[e] = v[e];
-    stream_store(a, reinterpret_cast<f16x8*>(p));
-  }
-  // dequantize layout: 2 chunks of 8 columns, 8i + 128m (16-byte stores, 256 contiguous bytes per row)
-  static constexpr int kDqChunks = 2, kDqWidth = 8;
-  __device__ static __forceinline__ void store_chunk(f16* p, const f16 (&v)[8]) { store8(p, v); }
-  __device__ static __forceinline__ float to_float(f16 v) { return (float)v; }
-  __device__ static __forceinline__ f16 from_float(float v) { return (f16)v; }
+  __device__ static __forceinline__ void set(Store& st, int k, int e, f16 x) { st.v[k][e >> 1][e & 1] = x; }
   __device__ static __forceinline__ float init_lo() { return __builtin_inff(); }  // half(1e30) is +inf
   __device__ static __forceinline__ float init_hi() { return -__builtin_inff(); }
+  __device__ static __forceinline__ f16 from_float(float v) { return (f16)v; }
+  __device__ static __forceinline__ void minmax(const Store& st, float& lo, float& hi) {
+    f16x2 l = {(f16)lo, (f16)lo}, h = {(f16)hi, (f16)hi};
+#pragma unroll
+    for (int k = 0; k < 2; k++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        l = __builtin_elementwise_min(l, st.v[k][j]);
+        h = __builtin_elementwise_max(h, st.v[k][j]);
+      }
+    lo = __builtin_fminf((float)l.x, (float)l.y);
+    hi = __builtin_fmaxf((float)h.x, (float)h.y);
+  }
   // range is a half operation; the quotient is a double narrowed to float and then to half
   __device__ static __forceinline__ f16 make_scale(f16 lo, f16 hi, int qmax) {
     f16 range = hi - lo;
     return (f16)(float)((double)(float)qmax / ((double)(float)range + 2e-6));
   }
-  // half subtraction and half product (each rounded to half), then float from there on
-  __device__ static __forceinline__ int code(f16 x, f16 mn, f16 s, float u) {
-    f16 t = x - mn;
+  // float(p) + u with p taken from the low / high half of a pair: one v_fma_mix_f32 (p * 1.0 + u)
+  __device__ static __forceinline__ float widen_add_lo(f16x2 p, float u) {
+    float y;
+    asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(y) : "v"(p), "v"(u));
+    return y;
+  }
+  __device__ static __forceinline__ float widen_add_hi(f16x2 p, float u) {
+    float y;
+    asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(y) : "v"(p), "v"(u));
+    return y;
+  }
+  // half subtraction and half product (each rounded to half), then float: y = float(p) + u,
+  // code = rint(max(y - 0.5, 0))
+  __device__ static __forceinline__ uint32_t code1(const Store& st, int k, int e, f16 mn, f16 s, float u) {
+    f16 t = st.v[k][e >> 1][e & 1] - mn;
     f16 p = t * s;
     float y = (float)p + u;
-    float z = __builtin_fmaxf(y - 0.5f, 0.0f);
-    return (int)__builtin_rintf(z);
+    return rint_clamp0(y - 0.5f);
   }
-  // half(code) / scale is a float division rounded to half; the sum is rounded to half again
-  __device__ static __forceinline__ f16 decode(int c, f16 s, f16 mn) {
-    f16 q = (f16)((float)c / (float)s);
-    return q + mn;
+  template <bool CONST_NOISE>
+  __device__ static __forceinline__ void codes8(const Store& st, int k, f16 mn, f16 s, const float (&u)[8],
+                                                uint32_t (&c)[8]) {
+    const f16x2 mn2 = {mn, mn}, s2 = {s, s};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      f16x2 t = st.v[k][j] - mn2;
+      f16x2 p = t * s2;
+      if (CONST_NOISE) {
+        // u = 0.5: float(p) + 0.5 and the following - 0.5 are both exact for every half p
+        // (at most 24 significant bits between 2^-1 and p's last bit), so y - 0.5 == float(p)
+        c[2 * j] = rint_clamp0((float)p.x);
+        c[2 * j + 1] = rint_clamp0((float)p.y);
+      } else {
+        c[2 * j] = rint_clamp0(widen_add_lo(p, u[2 * j]) - 0.5f);
+        c[2 * j + 1] = rint_clamp0(widen_add_hi(p, u[2 * j + 1]) - 0.5f);
+      }
+    }
+  }
+
+  // ---- dequantize: half(code) / scale is a float division rounded to half; the sum is rounded to half ----
+  struct Dq { float s, r; f16 mn; bool fast; };
+  __device__ static __forceinline__ Dq dq_prepare(f16 s, f16 mn) {
+    Dq d;
+    d.s = (float)s; d.mn = mn;
+    d.fast = reciprocal_safe(d.s);
+    d.r = 1.0f / d.s;
+    return d;
+  }
+  __device__ static __forceinline__ f16 decode(int c, const Dq& d) {
+    float q = d.fast ? div_by_reciprocal((float)c, d.s, d.r) : (float)c / d.s;
+    return (f16)q + d.mn;
+  }
+  static constexpr int kDqWidth = 8;  // columns per dequantize lane: one 16-byte store
+  __device__ static __forceinline__ void store_dq(f16* p, const f16 (&v)[8]) {
+    f16x8 a;
+#pragma unroll
+    for (int e = 0; e < 8; e++) a[e] = v[e];
+    stream_store(a, reinterpret_cast<f16x8*>(p));
   }
 };
 
-// Column of element e (0..7) of chunk k (0,1) for row lane i.
+// Column of the first element of chunk k (0,1) for row lane i.
 __device__ __forceinline__ int chunk_col(int k, int i) { return 128 * k + 8 * i; }
 
 // Load the 16 elements lane i owns of group n; elements at or beyond numel read as zero (the zero
 // padding of gact/gact/ops.py:12-17 without the copy).
 template <typename T>
 __device__ __forceinline__ void load_group(const T* __restrict__ x, int64_t numel, int64_t n, int i,
-                                           T (&v)[2][8]) {
+                                           typename Elem<T>::Store& st) {
   const int64_t base = n * GROUP;
   if (base + GROUP <= numel) {
 #pragma unroll
-    for (int k = 0; k < 2; k++) Elem<T>::load8(x + base + chunk_col(k, i), v[k]);
+    for (int k = 0; k < 2; k++) Elem<T>::load_chunk(x + base + chunk_col(k, i), st, k);
   } else {
 #pragma unroll
     for (int k = 0; k < 2; k++)
 #pragma unroll
       for (int e = 0; e < 8; e++) {
         int64_t idx = base + chunk_col(k, i) + e;
-        v[k][e] = idx < numel ? x[idx] : (T)0;
-      }
-  }
-}
-
-template <typename T>
-__device__ __forceinline__ void store_group(T* __restrict__ out, int64_t numel, int64_t n, int i,
-                                            const T (&v)[2][8]) {
-  const int64_t base = n * GROUP;
-  if (base + GROUP <= numel) {
-#pragma unroll
-    for (int k = 0; k < 2; k++) Elem<T>::store8(out + base + chunk_col(k, i), v[k]);
-  } else {
-#pragma unroll
-    for (int k = 0; k < 2; k++)
-#pragma unroll
-      for (int e = 0; e < 8; e++) {
-        int64_t idx = base + chunk_col(k, i) + e;
-        if (idx < numel) out[idx] = v[k][e];
+        Elem<T>::set(st, k, e, idx < numel ? x[idx] : (T)0);
       }
   }
 }
 
 // ------------------------------------------------------------------------------------------------
-// Quantize one super-group: the 8/BITS consecutive groups whose codes share output bytes.
+// Quantize one super-group (one 16-lane row).
 //   GIVEN = false: min/max are reduced here (fused minimax + scale + pack, one read of x).
 //   GIVEN = true : min/max are read from mn_io / mx_io (the pack entry point's contract).
-// Codes follow quantization_cuda_kernel.cu:38-71; see Elem<T>::code for the arithmetic.
+// Codes follow quantization_cuda_kernel.cu:38-71; see Elem<T>::code1 for the arithmetic.
 // ------------------------------------------------------------------------------------------------
 template <typename T, int BITS, int NOISE, bool GIVEN>
 __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int64_t numel, int64_t N, int64_t sg,
@@ -249,155 +333,150 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
                                                     const float* __restrict__ noise) {
   constexpr int WPT = 8 / BITS;
   constexpr int QMAX = (1 << BITS) - 1;
-  {
-    const int64_t n0 = sg * WPT;
-
-    T v[WPT][2][8];
-    T lo_t[WPT], s_t[WPT];
-#pragma unroll
-    for (int ni = 0; ni < WPT; ni++) {
-      if (n0 + ni < N) load_group<T>(x, numel, n0 + ni, i, v[ni]);
-    }
-#pragma unroll
-    for (int ni = 0; ni < WPT; ni++) {
-      const int64_t n = n0 + ni;
-      if (n < N) {
-        T lo_v, hi_v;
-        if (GIVEN) {
-          lo_v = mn_io[n];
-          hi_v = mx_io[n];
-        } else {
-          float lo = Elem<T>::init_lo(), hi = Elem<T>::init_hi();
-#pragma unroll
-          for (int k = 0; k < 2; k++)
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-              float f = Elem<T>::to_float(v[ni][k][e]);
-              lo = __builtin_fminf(lo, f);
-              hi = __builtin_fmaxf(hi, f);
-            }
-          lo = row_all_min(lo);
-          hi = row_all_max(hi);
-          lo_v = Elem<T>::from_float(lo);
-          hi_v = Elem<T>::from_float(hi);
-        }
-        T s = Elem<T>::make_scale(lo_v, hi_v, QMAX);
-        lo_t[ni] = lo_v;
-        s_t[ni] = s;
-        if (i == ni) {
-          scale_out[n] = s;
-          if (!GIVEN) {
-            mn_io[n] = lo_v;
-            if (mx_io) mx_io[n] = hi_v;
-          }
-        }
-      }
-    }
-
-    uint32_t bytes[2][8];
-#pragma unroll
-    for (int k = 0; k < 2; k++)
-#pragma unroll
-      for (int e = 0; e < 8; e++) bytes[k][e] = 0;
-
-    if (NOISE == GACT_NOISE_REF) {
-      // one Philox state per output byte j: key = seed, counter = (draw/4, 0, j lo, j hi)
-#pragma unroll
-      for (int k = 0; k < 2; k++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-          const uint64_t j = (uint64_t)sg * GROUP + chunk_col(k, i) + e;
-          uint32_t r[4];
-#pragma unroll
-          for (int ni = 0; ni < WPT; ni++) {
-            if ((ni & 3) == 0) philox4x32_10(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r);
-            if (n0 + ni < N) {
-              float u = curand_uniform_map(r[ni & 3]);
-              int c = Elem<T>::code(v[ni][k][e], lo_t[ni], s_t[ni], u);
-              bytes[k][e] |= (uint32_t)c << (ni * BITS);
-            }
-          }
-        }
-    } else {
-#pragma unroll
-      for (int ni = 0; ni < WPT; ni++) {
-        const int64_t n = n0 + ni;
-        if (n < N) {
-#pragma unroll
-          for (int k = 0; k < 2; k++) {
-            float u[8];
-            if (NOISE == GACT_NOISE_CONST) {
-#pragma unroll
-              for (int e = 0; e < 8; e++) u[e] = 0.5f;
-            } else if (NOISE == GACT_NOISE_INJECT) {
-              Elem<float>::load8(noise + n * GROUP + chunk_col(k, i), u);
-            } else {  // GACT_NOISE_FAST: block index = flat element index / 8
-              const uint64_t blk = (uint64_t)n * (GROUP / 8) + 16 * k + i;
-              uint32_t r[4];
-              philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
-#pragma unroll
-              for (int e = 0; e < 8; e++) u[e] = fast_uniform_map((e & 1) ? (r[e >> 1] >> 16) : (r[e >> 1] & 0xffffu));
-            }
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-              int c = Elem<T>::code(v[ni][k][e], lo_t[ni], s_t[ni], u[e]);
-              bytes[k][e] |= (uint32_t)c << (ni * BITS);
-            }
-          }
-        }
-      }
-    }
-
-    // the reference accumulates in a uint8_t: keep the low 8 bits of every byte, then 8 bytes per chunk
-#pragma unroll
-    for (int k = 0; k < 2; k++) {
-      u32x2 w;
-      w.x = (bytes[k][0] & 0xffu) | ((bytes[k][1] & 0xffu) << 8) | ((bytes[k][2] & 0xffu) << 16) | (bytes[k][3] << 24);
-      w.y = (bytes[k][4] & 0xffu) | ((bytes[k][5] & 0xffu) << 8) | ((bytes[k][6] & 0xffu) << 16) | (bytes[k][7] << 24);
-      stream_store(w, reinterpret_cast<u32x2*>(packed + sg * GROUP + chunk_col(k, i)));
-    }
-  }
-}
-
-// Dequantize one super-group.  quantization_cuda_kernel.cu:149-177.
-template <typename T, int BITS>
-__device__ __forceinline__ void dequantize_supergroup(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
-                                                      const T* __restrict__ mn, int64_t numel, int64_t N, int64_t sg,
-                                                      int i, T* __restrict__ out) {
-  constexpr int WPT = 8 / BITS;
-  constexpr int CH = Elem<T>::kDqChunks, W = Elem<T>::kDqWidth;  // chunk m covers columns W*i + 16*W*m .. +W-1
   const int64_t n0 = sg * WPT;
-  uint32_t w[CH][W / 4];
+
+  typename Elem<T>::Store v[WPT];
+  T lo_t[WPT], s_t[WPT];
 #pragma unroll
-  for (int m = 0; m < CH; m++) {
-    const uint8_t* p = packed + sg * GROUP + W * i + 16 * W * m;
-    if (W == 4) {
-      w[m][0] = stream_load(reinterpret_cast<const uint32_t*>(p));
-    } else {
-      u32x2 t = stream_load(reinterpret_cast<const u32x2*>(p));
-      w[m][0] = t.x;
-      w[m][W / 4 - 1] = t.y;
-    }
+  for (int ni = 0; ni < WPT; ni++) {
+    if (n0 + ni < N) load_group<T>(x, numel, n0 + ni, i, v[ni]);
   }
 #pragma unroll
   for (int ni = 0; ni < WPT; ni++) {
     const int64_t n = n0 + ni;
     if (n < N) {
-      const T s = scale[n];
-      const T mv = mn[n];
-      const int64_t base = n * GROUP;
-      const bool full = base + GROUP <= numel;
+      T lo_v, hi_v;
+      if (GIVEN) {
+        lo_v = mn_io[n];
+        hi_v = mx_io[n];
+      } else {
+        float lo = Elem<T>::init_lo(), hi = Elem<T>::init_hi();
+        Elem<T>::minmax(v[ni], lo, hi);
+        lo = row_all_min(lo);
+        hi = row_all_max(hi);
+        lo_v = Elem<T>::from_float(lo);
+        hi_v = Elem<T>::from_float(hi);
+      }
+      T s = Elem<T>::make_scale(lo_v, hi_v, QMAX);
+      lo_t[ni] = lo_v;
+      s_t[ni] = s;
+      if (i == ni) {
+        scale_out[n] = s;
+        if (!GIVEN) {
+          mn_io[n] = lo_v;
+          if (mx_io) mx_io[n] = hi_v;
+        }
+      }
+    }
+  }
+
+  uint32_t bytes[2][8];
 #pragma unroll
-      for (int m = 0; m < CH; m++) {
+  for (int k = 0; k < 2; k++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) bytes[k][e] = 0;
+
+  if (NOISE == GACT_NOISE_REF) {
+    // one Philox state per output byte j: key = seed, counter = (draw/4, 0, j lo, j hi)
+#pragma unroll
+    for (int k = 0; k < 2; k++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const uint64_t j = (uint64_t)sg * GROUP + chunk_col(k, i) + e;
+        uint32_t r[4];
+#pragma unroll
+        for (int ni = 0; ni < WPT; ni++) {
+          if ((ni & 3) == 0) philox4x32_10(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r);
+          if (n0 + ni < N) {
+            float u = curand_uniform_map(r[ni & 3]);
+            bytes[k][e] |= Elem<T>::code1(v[ni], k, e, lo_t[ni], s_t[ni], u) << (ni * BITS);
+          }
+        }
+      }
+  } else {
+#pragma unroll
+    for (int ni = 0; ni < WPT; ni++) {
+      const int64_t n = n0 + ni;
+      if (n < N) {
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+          float u[8];
+          if (NOISE == GACT_NOISE_CONST) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) u[e] = 0.5f;
+          } else if (NOISE == GACT_NOISE_INJECT) {
+            Elem<float>::load8(noise + n * GROUP + chunk_col(k, i), u);
+          } else {  // GACT_NOISE_FAST: block index = flat element index / 8
+            const uint64_t blk = (uint64_t)n * (GROUP / 8) + 16 * k + i;
+            uint32_t r[4];
+            philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
+#pragma unroll
+            for (int e = 0; e < 8; e++) u[e] = fast_uniform_map((e & 1) ? (r[e >> 1] >> 16) : (r[e >> 1] & 0xffffu));
+          }
+          uint32_t c[8];
+          Elem<T>::template codes8<NOISE == GACT_NOISE_CONST>(v[ni], k, lo_t[ni], s_t[ni], u, c);
+#pragma unroll
+          for (int e = 0; e < 8; e++) bytes[k][e] |= c[e] << (ni * BITS);
+        }
+      }
+    }
+  }
+
+  // the reference accumulates in a uint8_t: keep the low 8 bits of every byte, then 8 bytes per chunk
+#pragma unroll
+  for (int k = 0; k < 2; k++) {
+    u32x2 w;
+    w.x = (bytes[k][0] & 0xffu) | ((bytes[k][1] & 0xffu) << 8) | ((bytes[k][2] & 0xffu) << 16) | (bytes[k][3] << 24);
+    w.y = (bytes[k][4] & 0xffu) | ((bytes[k][5] & 0xffu) << 8) | ((bytes[k][6] & 0xffu) << 16) | (bytes[k][7] << 24);
+    stream_store(w, reinterpret_cast<u32x2*>(packed + sg * GROUP + chunk_col(k, i)));
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Dequantize a unit of 8 consecutive groups (BITS super-groups).  A lane owns the W = 16/sizeof(T)
+// columns W*l .. W*l+W-1 of every group (one 16-byte store per group), so 256/W lanes cover a group:
+// a whole wave per unit for float, half a wave for half.  All code words are loaded first, then the 8
+// groups are written, each store instruction covering whole groups contiguously.
+// quantization_cuda_kernel.cu:149-177.
+// ------------------------------------------------------------------------------------------------
+template <typename T, int BITS>
+__device__ __forceinline__ void dequantize_8groups(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
+                                                   const T* __restrict__ mn, int64_t numel, int64_t N, int64_t unit,
+                                                   int l, T* __restrict__ out) {
+  constexpr int WPT = 8 / BITS;
+  constexpr int W = Elem<T>::kDqWidth;
+  const int64_t sg0 = unit * BITS;
+  const int64_t n_sg = (N + WPT - 1) / WPT;
+  uint32_t w[BITS][W / 4];
+#pragma unroll
+  for (int it = 0; it < BITS; it++) {
+    const uint8_t* p = packed + (sg0 + it) * GROUP + W * l;
+    const bool live = sg0 + it < n_sg;
+    if (W == 4) {
+      w[it][0] = live ? stream_load(reinterpret_cast<const uint32_t*>(p)) : 0u;
+    } else {
+      u32x2 t = {0u, 0u};
+      if (live) t = stream_load(reinterpret_cast<const u32x2*>(p));
+      w[it][0] = t.x;
+      w[it][W / 4 - 1] = t.y;
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < BITS; it++) {
+#pragma unroll
+    for (int ni = 0; ni < WPT; ni++) {
+      const int64_t n = (sg0 + it) * WPT + ni;
+      if (n < N) {
+        const typename Elem<T>::Dq d = Elem<T>::dq_prepare(scale[n], mn[n]);
         T v[W];
 #pragma unroll
         for (int e = 0; e < W; e++) {
-          int c = (int)__builtin_amdgcn_ubfe(w[m][e >> 2], 8 * (e & 3) + ni * BITS, BITS);
-          v[e] = Elem<T>::decode(c, s, mv);
+          int c = (int)__builtin_amdgcn_ubfe(w[it][e >> 2], 8 * (e & 3) + ni * BITS, BITS);
+          v[e] = Elem<T>::decode(c, d);
         }
-        const int64_t at = base + W * i + 16 * W * m;
-        if (full) {
-          Elem<T>::store_chunk(out + at, v);
+        const int64_t at = n * GROUP + W * l;
+        if (n * GROUP + GROUP <= numel) {
+          Elem<T>::store_dq(out + at, v);
         } else {
 #pragma unroll
           for (int e = 0; e < W; e++)
@@ -423,16 +502,18 @@ __device__ __forceinline__ void quantize_row(const T* __restrict__ x, int64_t nu
                                                (uint32_t)(seed >> 32), noise);
   }
 }
+// A wave of the batched dequantize owns 32 consecutive groups (four units of 8); with half a wave per
+// unit (half tensors) the two halves take alternate units.
 template <typename T, int BITS>
-__device__ __forceinline__ void dequantize_row(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
-                                               const T* __restrict__ mn, int64_t numel, int64_t N, int64_t row,
-                                               int i, T* __restrict__ out) {
-  constexpr int WPT = 8 / BITS;
+__device__ __forceinline__ void dequantize_wave32(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
+                                                  const T* __restrict__ mn, int64_t numel, int64_t N, int64_t wave,
+                                                  int lane, T* __restrict__ out) {
+  constexpr int LPU = GROUP / Elem<T>::kDqWidth;  // lanes per unit
+  constexpr int UPW = 64 / LPU;                   // units a wave works on at a time
 #pragma unroll 1
-  for (int it = 0; it < BITS; it++) {
-    const int64_t sg = row * BITS + it;
-    if (sg * WPT >= N) break;
-    dequantize_supergroup<T, BITS>(packed, scale, mn, numel, N, sg, i, out);
+  for (int it = 0; it < 4 / UPW; it++) {
+    const int64_t unit = wave * 4 + it * UPW + lane / LPU;
+    if (unit * ROW_GROUPS < N) dequantize_8groups<T, BITS>(packed, scale, mn, numel, N, unit, lane % LPU, out);
   }
 }
 
@@ -444,17 +525,10 @@ __device__ __forceinline__ void minimax_row(const T* __restrict__ x, int64_t N, 
   for (int g = 0; g < ROW_GROUPS; g++) {
     const int64_t n = row * ROW_GROUPS + g;
     if (n >= N) break;
-    T v[2][8];
+    typename Elem<T>::Store v;
     load_group<T>(x, N * GROUP, n, i, v);
     float lo = Elem<T>::init_lo(), hi = Elem<T>::init_hi();
-#pragma unroll
-    for (int k = 0; k < 2; k++)
-#pragma unroll
-      for (int e = 0; e < 8; e++) {
-        float f = Elem<T>::to_float(v[k][e]);
-        lo = __builtin_fminf(lo, f);
-        hi = __builtin_fmaxf(hi, f);
-      }
+    Elem<T>::minmax(v, lo, hi);
     lo = row_all_min(lo);
     hi = row_all_max(hi);
     if (i == 0) {
@@ -482,9 +556,10 @@ template <typename T, int BITS>
 __global__ void __launch_bounds__(256)
 dequantize_kernel(const uint8_t* __restrict__ packed, const T* __restrict__ scale, const T* __restrict__ mn,
                   int64_t numel, int64_t N, T* __restrict__ out) {
-  const int64_t sg = (int64_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
-  if (sg * (8 / BITS) >= N) return;
-  dequantize_supergroup<T, BITS>(packed, scale, mn, numel, N, sg, threadIdx.x & 15, out);
+  constexpr int LPU = GROUP / Elem<T>::kDqWidth;  // lanes per unit of 8 groups: 64 (float) or 32 (half)
+  const int64_t unit = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / LPU;
+  if (unit * ROW_GROUPS >= N) return;
+  dequantize_8groups<T, BITS>(packed, scale, mn, numel, N, unit, threadIdx.x % LPU, out);
 }
 
 template <typename T>
@@ -508,7 +583,7 @@ minimax_any_kernel(const T* __restrict__ x, int64_t N, int64_t D, T* __restrict_
   const int lane = threadIdx.x & 63;
   float lo = Elem<T>::init_lo(), hi = Elem<T>::init_hi();
   for (int64_t d = lane; d < D; d += 64) {
-    float f = Elem<T>::to_float(x[n * D + d]);
+    float f = (float)x[n * D + d];
     lo = __builtin_fminf(lo, f);
     hi = __builtin_fmaxf(hi, f);
   }
@@ -562,8 +637,9 @@ pack_any_kernel(const T* __restrict__ data, const T* __restrict__ mn, const T* _
       const int e = (int)(id & 7);
       u = fast_uniform_map((e & 1) ? (r[e >> 1] >> 16) : (r[e >> 1] & 0xffffu));
     }
-    int c = Elem<T>::code(data[id], mn[sid], scale[sid], u);
-    byte |= (uint32_t)c << (ni * bits);
+    typename Elem<T>::Store one;
+    Elem<T>::set(one, 0, 0, data[id]);
+    byte |= Elem<T>::code1(one, 0, 0, mn[sid], scale[sid], u) << (ni * bits);
   }
   packed[j] = (uint8_t)byte;
 }
@@ -585,7 +661,7 @@ unpack_any_kernel(const uint8_t* __restrict__ packed, int bits, const T* __restr
     if (n >= N) break;
     const int64_t sid = n * G + g;
     int c = (int)((byte >> (ni * bits)) & ((1u << bits) - 1u));
-    out[(n * G + g) * D + d] = Elem<T>::decode(c, scale[sid], mn[sid]);
+    out[(n * G + g) * D + d] = Elem<T>::decode(c, Elem<T>::dq_prepare(scale[sid], mn[sid]));
   }
 }
 
@@ -801,13 +877,13 @@ dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int3
   const gact_batch_entry ent = table[t];
   const int bt = bits[t];
   const int64_t N = (ent.numel + GROUP - 1) / GROUP;
-  const int64_t row = ((int64_t)blockIdx.x - ent.first_block) * 16 + (threadIdx.x >> 4);
-  if (row * ROW_GROUPS >= N) return;
-  const int i = threadIdx.x & 15;
+  const int64_t wave = ((int64_t)blockIdx.x - ent.first_block) * 4 + (threadIdx.x >> 6);  // 32 groups per wave
+  if (wave * 32 >= N) return;
+  const int i = threadIdx.x & 63;
   const uint8_t* packed = packed_arena + ent.packed_offset;
   const uint8_t* sc = scale_arena + ent.stats_offset * 4;
   const uint8_t* mn = min_arena + ent.stats_offset * 4;
-#define GACT_DB(T, B) dequantize_row<T, B>(packed, (const T*)sc, (const T*)mn, ent.numel, N, row, i, (T*)ent.x)
+#define GACT_DB(T, B) dequantize_wave32<T, B>(packed, (const T*)sc, (const T*)mn, ent.numel, N, wave, i, (T*)ent.x)
   if (ent.dtype == GACT_F32) {
     switch (bt) {
       case 1: GACT_DB(float, 1); break;
@@ -886,8 +962,9 @@ int dispatch_quantize(int bits, const T* x, int64_t numel, int64_t N, uint8_t* p
 template <typename T>
 int dispatch_dequantize(int bits, const uint8_t* packed, const T* scale, const T* mn, int64_t numel, int64_t N, T* out,
                         hipStream_t stream) {
-  dim3 grid, block;
-  row_grid(supergroups(N, bits), &grid, &block);
+  // a unit of 8 groups takes 256 / (16 / sizeof(T)) lanes
+  const int64_t units_per_block = 256 / (GROUP / (16 / (int64_t)sizeof(T)));
+  const dim3 grid((unsigned)(((N + ROW_GROUPS - 1) / ROW_GROUPS + units_per_block - 1) / units_per_block)), block(256);
   switch (bits) {
     case 1: hipLaunchKernelGGL((dequantize_kernel<T, 1>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
     case 2: hipLaunchKernelGGL((dequantize_kernel<T, 2>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
