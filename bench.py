@@ -26,8 +26,12 @@ for _p in (ROOT, os.path.join(ROOT, "gact-icml_amd")):
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
-# a copy kernel of known size (see profiles/); None until measured for the workload
-TRAFFIC_BYTES = {}
+# a copy kernel of known size (profiles/config2_fp32_4bit_quantize_dequantize.txt: the copy kernel reads
+# FETCH_SIZE x 1.99988 and WRITE_SIZE x 1.00000 KiB); None for workloads without a counter run
+TRAFFIC_BYTES = {
+    ("config2", "quantize"): 473.8e6,    # 419.2 MB read + 54.6 MB written; algorithmic 465.6 MB
+    ("config2", "dequantize"): 465.9e6,  # 54.7 MB read + 411.1 MB written; algorithmic 465.6 MB
+}
 
 WORKLOADS = {
     # name: (shape, dtype, bits, rng_stream, data kind, description)
@@ -160,6 +164,9 @@ def main():
     ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS))
     ap.add_argument("--all", action="store_true", help="also time the other single-tensor workloads (extra key)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="after the timed region also launch 20 plain device copies of the workload tensor, so "
+                         "that a counter run of this command holds a copy kernel of known size to scale by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no cross-GPU step (each rank compresses its own "
@@ -186,6 +193,15 @@ def main():
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get((args.workload, dom))},
     }
+    if args.copy_calibration:
+        y = torch.empty_like(x)
+        for _ in range(20):
+            y.copy_(x)
+        torch.cuda.synchronize()
+        line["copy_calibration"] = {"kernel": "torch elementwise copy", "launches": 20,
+                                    "bytes_read": x.numel() * x.element_size(),
+                                    "bytes_written": x.numel() * x.element_size()}
+        del y
     if args.all:
         extra = []
         for name in sorted(WORKLOADS):
