@@ -149,26 +149,32 @@ __device__ __forceinline__ bool reciprocal_safe(float s) {
 template <typename T> struct Elem;
 
 template <> struct Elem<float> {
-  struct Store { float v[2][8]; };
-  __device__ static __forceinline__ void load8(const float* p, float (&v)[8]) {
+  // quantize layout: 4 chunks of 4 columns, 4i + 64m: one 16-byte load per chunk, 256 contiguous
+  // bytes per row and load instruction
+  static constexpr int kQChunks = 4, kQWidth = 4;
+  struct Store { float v[4][4]; };
+  __device__ static __forceinline__ void load_noise(const float* p, float (&u)[4]) {
     f32x4 a = stream_load(reinterpret_cast<const f32x4*>(p));
-    f32x4 b = stream_load(reinterpret_cast<const f32x4*>(p + 4));
-    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    u[0] = a.x; u[1] = a.y; u[2] = a.z; u[3] = a.w;
   }
-  __device__ static __forceinline__ void load_chunk(const float* p, Store& st, int k) { load8(p, st.v[k]); }
+  __device__ static __forceinline__ void load_chunk(const float* p, Store& st, int k) { load_noise(p, st.v[k]); }
   __device__ static __forceinline__ void set(Store& st, int k, int e, float x) { st.v[k][e] = x; }
   __device__ static __forceinline__ float init_lo() { return 1e30f; }
   __device__ static __forceinline__ float init_hi() { return -1e30f; }
   __device__ static __forceinline__ float from_float(float v) { return v; }
   __device__ static __forceinline__ void minmax(const Store& st, float& lo, float& hi) {
 #pragma unroll
-    for (int k = 0; k < 2; k++)
+    for (int k = 0; k < 4; k++)
 #pragma unroll
-      for (int e = 0; e < 8; e++) {
+      for (int e = 0; e < 4; e++) {
         lo = __builtin_fminf(lo, st.v[k][e]);
         hi = __builtin_fmaxf(hi, st.v[k][e]);
       }
+  }
+  __device__ static __forceinline__ void store_codes(uint8_t* p, const uint32_t (&b)[4]) {
+    // the reference accumulates in a uint8_t: keep the low 8 bits of every byte
+    uint32_t w = (b[0] & 0xffu) | ((b[1] & 0xffu) << 8) | ((b[2] & 0xffu) << 16) | (b[3] << 24);
+    stream_store(w, reinterpret_cast<uint32_t*>(p));
   }
   // scale = float( double(float(qmax)) / (double(max - min) + 2e-6) )
   __device__ static __forceinline__ float make_scale(float lo, float hi, int qmax) {
@@ -182,10 +188,10 @@ template <> struct Elem<float> {
     return rint_clamp0(y - 0.5f);
   }
   template <bool CONST_NOISE>
-  __device__ static __forceinline__ void codes8(const Store& st, int k, float mn, float s, const float (&u)[8],
-                                                uint32_t (&c)[8]) {
+  __device__ static __forceinline__ void codes(const Store& st, int k, float mn, float s, const float (&u)[4],
+                                               uint32_t (&c)[4]) {
 #pragma unroll
-    for (int e = 0; e < 8; e++) c[e] = code1(st, k, e, mn, s, u[e]);
+    for (int e = 0; e < 4; e++) c[e] = code1(st, k, e, mn, s, u[e]);
   }
 
   // ---- dequantize: out = float(code) / scale + min ----
@@ -209,7 +215,21 @@ template <> struct Elem<float> {
 };
 
 template <> struct Elem<f16> {
+  // quantize layout: 2 chunks of 8 columns, 8i + 128m: one 16-byte load per chunk
+  static constexpr int kQChunks = 2, kQWidth = 8;
   struct Store { f16x2 v[2][4]; };   // pairs, so that subtraction and product run as packed ops
+  __device__ static __forceinline__ void store_codes(uint8_t* p, const uint32_t (&b)[8]) {
+    u32x2 w;
+    w.x = (b[0] & 0xffu) | ((b[1] & 0xffu) << 8) | ((b[2] & 0xffu) << 16) | (b[3] << 24);
+    w.y = (b[4] & 0xffu) | ((b[5] & 0xffu) << 8) | ((b[6] & 0xffu) << 16) | (b[7] << 24);
+    stream_store(w, reinterpret_cast<u32x2*>(p));
+  }
+  __device__ static __forceinline__ void load_noise(const float* p, float (&u)[8]) {
+    f32x4 a = stream_load(reinterpret_cast<const f32x4*>(p));
+    f32x4 b = stream_load(reinterpret_cast<const f32x4*>(p + 4));
+    u[0] = a.x; u[1] = a.y; u[2] = a.z; u[3] = a.w;
+    u[4] = b.x; u[5] = b.y; u[6] = b.z; u[7] = b.w;
+  }
   __device__ static __forceinline__ void load_chunk(const f16* p, Store& st, int k) {
     f16x8 a = stream_load(reinterpret_cast<const f16x8*>(p));
 #pragma unroll
@@ -256,8 +276,8 @@ template <> struct Elem<f16> {
     return rint_clamp0(y - 0.5f);
   }
   template <bool CONST_NOISE>
-  __device__ static __forceinline__ void codes8(const Store& st, int k, f16 mn, f16 s, const float (&u)[8],
-                                                uint32_t (&c)[8]) {
+  __device__ static __forceinline__ void codes(const Store& st, int k, f16 mn, f16 s, const float (&u)[8],
+                                               uint32_t (&c)[8]) {
     const f16x2 mn2 = {mn, mn}, s2 = {s, s};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -297,26 +317,77 @@ template <> struct Elem<f16> {
   }
 };
 
-// Column of the first element of chunk k (0,1) for row lane i.
-__device__ __forceinline__ int chunk_col(int k, int i) { return 128 * k + 8 * i; }
+// Column of the first element of chunk k for row lane i: chunks are W columns wide and 16*W apart.
+template <typename T>
+__device__ __forceinline__ int chunk_col(int k, int i) { return Elem<T>::kQWidth * (16 * k + i); }
 
 // Load the 16 elements lane i owns of group n; elements at or beyond numel read as zero (the zero
 // padding of gact/gact/ops.py:12-17 without the copy).
 template <typename T>
 __device__ __forceinline__ void load_group(const T* __restrict__ x, int64_t numel, int64_t n, int i,
                                            typename Elem<T>::Store& st) {
+  constexpr int CH = Elem<T>::kQChunks, W = Elem<T>::kQWidth;
   const int64_t base = n * GROUP;
   if (base + GROUP <= numel) {
 #pragma unroll
-    for (int k = 0; k < 2; k++) Elem<T>::load_chunk(x + base + chunk_col(k, i), st, k);
+    for (int k = 0; k < CH; k++) Elem<T>::load_chunk(x + base + chunk_col<T>(k, i), st, k);
   } else {
 #pragma unroll
-    for (int k = 0; k < 2; k++)
+    for (int k = 0; k < CH; k++)
 #pragma unroll
-      for (int e = 0; e < 8; e++) {
-        int64_t idx = base + chunk_col(k, i) + e;
+      for (int e = 0; e < W; e++) {
+        int64_t idx = base + chunk_col<T>(k, i) + e;
         Elem<T>::set(st, k, e, idx < numel ? x[idx] : (T)0);
       }
+  }
+}
+
+// 16-bit piece e of a pair of Philox words -> uniform of the fast stream
+__device__ __forceinline__ float fast_piece(uint32_t w0, uint32_t w1, int e) {
+  const uint32_t w = (e & 2) ? w1 : w0;
+  return fast_uniform_map((e & 1) ? (w >> 16) : (w & 0xffffu));
+}
+// swap with the neighbouring lane (lane ^ 1): DPP quad_perm [1,0,3,2]
+__device__ __forceinline__ uint32_t swap_with_neighbour(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0xB1, 0xf, 0xf, false);
+}
+
+// The fast stream's uniforms for all chunks of group n that lane i owns.  One Philox block feeds 8
+// consecutive elements.  With 8-column chunks that is one block per chunk; with 4-column chunks two
+// neighbouring lanes share a block, so the even lane computes the block of chunk m, the odd lane the
+// block of chunk m+1, and they exchange the halves the other one needs.
+template <typename T>
+__device__ __forceinline__ void fast_noise(int64_t n, int i, uint32_t k0, uint32_t k1,
+                                           float (&u)[Elem<T>::kQChunks][Elem<T>::kQWidth]) {
+  constexpr int CH = Elem<T>::kQChunks, W = Elem<T>::kQWidth;
+  if (W == 8) {
+#pragma unroll
+    for (int k = 0; k < CH; k++) {
+      const uint64_t blk = (uint64_t)n * (GROUP / 8) + 16 * k + i;
+      uint32_t r[4];
+      philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
+#pragma unroll
+      for (int e = 0; e < W; e++) u[k][e] = fast_piece(r[(e >> 2) * 2], r[(e >> 2) * 2 + 1], e & 3);
+    }
+  } else {
+    const bool odd = i & 1;
+#pragma unroll
+    for (int m = 0; m < CH; m += 2) {
+      // element block of (chunk, lane): (4*(16*chunk + lane)) / 8 = 8*chunk + lane/2
+      const uint64_t blk = (uint64_t)n * (GROUP / 8) + 8 * (m + (odd ? 1 : 0)) + (i >> 1);
+      uint32_t r[4];
+      philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
+      // the even lane owns elements 0..3 of a block (words 0,1), the odd lane elements 4..7 (words 2,3)
+      const uint32_t ga = swap_with_neighbour(odd ? r[0] : r[2]);
+      const uint32_t gb = swap_with_neighbour(odd ? r[1] : r[3]);
+      const uint32_t a0 = odd ? ga : r[0], a1 = odd ? gb : r[1];   // chunk m
+      const uint32_t b0 = odd ? r[2] : ga, b1 = odd ? r[3] : gb;   // chunk m + 1
+#pragma unroll
+      for (int e = 0; e < W; e++) {
+        u[m][e] = fast_piece(a0, a1, e);
+        u[m + 1][e] = fast_piece(b0, b1, e);
+      }
+    }
   }
 }
 
@@ -333,6 +404,7 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
                                                     const float* __restrict__ noise) {
   constexpr int WPT = 8 / BITS;
   constexpr int QMAX = (1 << BITS) - 1;
+  constexpr int CH = Elem<T>::kQChunks, W = Elem<T>::kQWidth;
   const int64_t n0 = sg * WPT;
 
   typename Elem<T>::Store v[WPT];
@@ -370,19 +442,19 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
     }
   }
 
-  uint32_t bytes[2][8];
+  uint32_t bytes[CH][W];
 #pragma unroll
-  for (int k = 0; k < 2; k++)
+  for (int k = 0; k < CH; k++)
 #pragma unroll
-    for (int e = 0; e < 8; e++) bytes[k][e] = 0;
+    for (int e = 0; e < W; e++) bytes[k][e] = 0;
 
   if (NOISE == GACT_NOISE_REF) {
     // one Philox state per output byte j: key = seed, counter = (draw/4, 0, j lo, j hi)
 #pragma unroll
-    for (int k = 0; k < 2; k++)
+    for (int k = 0; k < CH; k++)
 #pragma unroll
-      for (int e = 0; e < 8; e++) {
-        const uint64_t j = (uint64_t)sg * GROUP + chunk_col(k, i) + e;
+      for (int e = 0; e < W; e++) {
+        const uint64_t j = (uint64_t)sg * GROUP + chunk_col<T>(k, i) + e;
         uint32_t r[4];
 #pragma unroll
         for (int ni = 0; ni < WPT; ni++) {
@@ -398,38 +470,33 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
     for (int ni = 0; ni < WPT; ni++) {
       const int64_t n = n0 + ni;
       if (n < N) {
+        float u[CH][W];
+        if (NOISE == GACT_NOISE_FAST) {
+          fast_noise<T>(n, i, k0, k1, u);
+        } else {
 #pragma unroll
-        for (int k = 0; k < 2; k++) {
-          float u[8];
-          if (NOISE == GACT_NOISE_CONST) {
+          for (int k = 0; k < CH; k++) {
+            if (NOISE == GACT_NOISE_INJECT) {
+              Elem<T>::load_noise(noise + n * GROUP + chunk_col<T>(k, i), u[k]);
+            } else {
 #pragma unroll
-            for (int e = 0; e < 8; e++) u[e] = 0.5f;
-          } else if (NOISE == GACT_NOISE_INJECT) {
-            Elem<float>::load8(noise + n * GROUP + chunk_col(k, i), u);
-          } else {  // GACT_NOISE_FAST: block index = flat element index / 8
-            const uint64_t blk = (uint64_t)n * (GROUP / 8) + 16 * k + i;
-            uint32_t r[4];
-            philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
-#pragma unroll
-            for (int e = 0; e < 8; e++) u[e] = fast_uniform_map((e & 1) ? (r[e >> 1] >> 16) : (r[e >> 1] & 0xffffu));
+              for (int e = 0; e < W; e++) u[k][e] = 0.5f;
+            }
           }
-          uint32_t c[8];
-          Elem<T>::template codes8<NOISE == GACT_NOISE_CONST>(v[ni], k, lo_t[ni], s_t[ni], u, c);
+        }
 #pragma unroll
-          for (int e = 0; e < 8; e++) bytes[k][e] |= c[e] << (ni * BITS);
+        for (int k = 0; k < CH; k++) {
+          uint32_t c[W];
+          Elem<T>::template codes<NOISE == GACT_NOISE_CONST>(v[ni], k, lo_t[ni], s_t[ni], u[k], c);
+#pragma unroll
+          for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (ni * BITS);
         }
       }
     }
   }
 
-  // the reference accumulates in a uint8_t: keep the low 8 bits of every byte, then 8 bytes per chunk
 #pragma unroll
-  for (int k = 0; k < 2; k++) {
-    u32x2 w;
-    w.x = (bytes[k][0] & 0xffu) | ((bytes[k][1] & 0xffu) << 8) | ((bytes[k][2] & 0xffu) << 16) | (bytes[k][3] << 24);
-    w.y = (bytes[k][4] & 0xffu) | ((bytes[k][5] & 0xffu) << 8) | ((bytes[k][6] & 0xffu) << 16) | (bytes[k][7] << 24);
-    stream_store(w, reinterpret_cast<u32x2*>(packed + sg * GROUP + chunk_col(k, i)));
-  }
+  for (int k = 0; k < CH; k++) Elem<T>::store_codes(packed + sg * GROUP + chunk_col<T>(k, i), bytes[k]);
 }
 
 // ------------------------------------------------------------------------------------------------
