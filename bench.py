@@ -121,6 +121,85 @@ def run_workload(torch, name, steps, warmup, seed=42):
     return res, x
 
 
+def run_config5(torch, steps, warmup, seed=42):
+    """BASELINE config 5, the full adaptive step: 120 fp16 tensors with Swin-Tiny-like shapes, per-tensor
+    sensitivities ~LogNormal(0,2), budget 2 bits per element.  One step = greedy calc_precision on the GPU
+    (widths stay in device memory), offset planning, one batched mixed-width quantize and one batched
+    dequantize, all through the C ABI."""
+    import numpy as np
+
+    from gact.batched import BatchedQuantizer
+    from gact.cpp_extension import _abi
+
+    lib = _abi.lib()
+    shapes = [(128, 3136, 96)] * 20 + [(128, 784, 192)] * 20 + [(128, 196, 384)] * 60 + [(128, 49, 768)] * 20
+    g = torch.Generator(device="cuda").manual_seed(0)
+    xs = [torch.randn(s, generator=g, device="cuda", dtype=torch.float16) for s in shapes]
+    outs = [torch.empty_like(x) for x in xs]
+    L = len(xs)
+    rng = np.random.default_rng(0)
+    C = torch.from_numpy(np.exp(rng.normal(0.0, 2.0, L)).astype(np.float32)).cuda()
+    w = torch.tensor([x.numel() for x in xs], dtype=torch.int64, device="cuda")
+    target = 2.0 * float(sum(x.numel() for x in xs))
+    init = torch.full((L,), 8, dtype=torch.int32, device="cuda")
+    bits = init.clone()
+    status = torch.zeros((1,), dtype=torch.int32, device="cuda")
+    bq = BatchedQuantizer([x.numel() for x in xs], [torch.float16] * L, "cuda")
+    seeds = [i + seed for i in range(L)]
+    table_q = bq._table(xs, seeds)
+    table_d = bq._table(outs, seeds)
+    packed = torch.empty((bq.arena_bytes_for_budget(target),), dtype=torch.uint8, device="cuda")
+    sc = torch.empty((bq.total_groups * 4,), dtype=torch.uint8, device="cuda")
+    mn = torch.empty((bq.total_groups * 4,), dtype=torch.uint8, device="cuda")
+    plan = torch.empty((2,), dtype=torch.int64, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+
+    def allocate():
+        bits.copy_(init)
+        _abi.check(lib.gact_calc_precision_device(bits.data_ptr(), C.data_ptr(), w.data_ptr(), L, target,
+                                                  status.data_ptr(), st))
+
+    def quantize():
+        _abi.check(lib.gact_batch_plan(table_q.data_ptr(), bits.data_ptr(), L, packed.numel(), plan.data_ptr(), st))
+        _abi.check(lib.gact_quantize_batched(table_q.data_ptr(), bits.data_ptr(), L, bq.total_blocks, _abi.NOISE_FAST,
+                                             plan.data_ptr(), packed.data_ptr(), sc.data_ptr(), mn.data_ptr(), st))
+
+    def dequantize():
+        _abi.check(lib.gact_batch_plan(table_d.data_ptr(), bits.data_ptr(), L, packed.numel(), plan.data_ptr(), st))
+        _abi.check(lib.gact_dequantize_batched(table_d.data_ptr(), bits.data_ptr(), L, bq.total_blocks,
+                                               plan.data_ptr(), packed.data_ptr(), sc.data_ptr(), mn.data_ptr(), st))
+
+    for _ in range(warmup):
+        allocate(); quantize(); dequantize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        ev[k][0].record(); allocate()
+        ev[k][1].record(); quantize()
+        ev[k][2].record(); dequantize()
+        ev[k][3].record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    host_bits = bits.cpu().tolist()
+    assert status.item() == 0 and plan.cpu().tolist()[1] == 1
+    per_dir = sum(algorithmic_bytes(x.numel(), 2, b) for x, b in zip(xs, host_bits))
+    a_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / steps
+    q_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / steps
+    d_ms = sum(e[2].elapsed_time(e[3]) for e in ev) / steps
+    wall_ms = (t1 - t0) * 1e3 / steps
+    return {
+        "workload": "config5", "desc": "120 fp16 Swin-Tiny-like tensors, widths by calc_precision on the GPU (budget "
+                                       "2 bits/element), one batched mixed-width quantize + dequantize",
+        "tensors": L, "elements": int(sum(x.numel() for x in xs)), "dtype": "float16", "rng_stream": "fast",
+        "width_histogram": {str(b): host_bits.count(b) for b in (1, 2, 4, 8)},
+        "bytes_per_direction": per_dir, "ms_per_step": wall_ms, "gbs": 2 * per_dir / (wall_ms * 1e-3) / 1e9,
+        "calc_precision": {"ms": a_ms},
+        "quantize": {"ms": q_ms, "gbs": per_dir / (q_ms * 1e-3) / 1e9},
+        "dequantize": {"ms": d_ms, "gbs": per_dir / (d_ms * 1e-3) / 1e9},
+    }
+
+
 def cpu_baseline(torch, x, bits, stream, budget_s=12.0):
     """The C restatement on the host cores over a leading slice of the same tensor."""
     import numpy as np
@@ -210,6 +289,8 @@ def main():
             r, _ = run_workload(torch, name, max(20, args.steps // 4), max(3, args.warmup // 4))
             extra.append(r)
             torch.cuda.empty_cache()
+        extra.append(run_config5(torch, 20, 3))
+        torch.cuda.empty_cache()
         line["other_workloads"] = extra
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(torch, x, res["bits"], res["rng_stream"])

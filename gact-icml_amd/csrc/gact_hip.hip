@@ -554,33 +554,36 @@ __device__ __forceinline__ void dequantize_8groups(const uint8_t* __restrict__ p
   }
 }
 
-// The 8 groups (BITS super-groups) of one row, one after the other: the batched launch, whose grid must
-// not depend on the widths.
-template <typename T, int BITS, int NOISE, bool GIVEN>
-__device__ __forceinline__ void quantize_row(const T* __restrict__ x, int64_t numel, int64_t N, int64_t row, int i,
-                                             uint8_t* __restrict__ packed, T* __restrict__ scale_out, T* mn_io,
-                                             T* mx_io, uint64_t seed, const float* __restrict__ noise) {
+// Batched launch: a block owns 128 consecutive groups of one tensor whatever the width, so the grid does
+// not depend on the widths.  Quantize: the 16*BITS super-groups of the block go round-robin over the 16
+// rows, so that every pass of the block reads one contiguous stretch.
+template <typename T, int BITS, int NOISE>
+__device__ __forceinline__ void quantize_block128(const T* __restrict__ x, int64_t numel, int64_t N, int64_t lb,
+                                                  uint8_t* __restrict__ packed, T* __restrict__ scale_out,
+                                                  T* __restrict__ mn_out, uint64_t seed) {
   constexpr int WPT = 8 / BITS;
+  const int row = threadIdx.x >> 4, i = threadIdx.x & 15;
 #pragma unroll 1
   for (int it = 0; it < BITS; it++) {
-    const int64_t sg = row * BITS + it;
-    if (sg * WPT >= N) break;
-    quantize_supergroup<T, BITS, NOISE, GIVEN>(x, numel, N, sg, i, packed, scale_out, mn_io, mx_io, (uint32_t)seed,
-                                               (uint32_t)(seed >> 32), noise);
+    const int64_t sg = lb * (16 * BITS) + it * 16 + row;
+    if (sg * WPT < N)
+      quantize_supergroup<T, BITS, NOISE, false>(x, numel, N, sg, i, packed, scale_out, mn_out, (T*)nullptr,
+                                                 (uint32_t)seed, (uint32_t)(seed >> 32), nullptr);
   }
 }
-// A wave of the batched dequantize owns 32 consecutive groups (four units of 8); with half a wave per
-// unit (half tensors) the two halves take alternate units.
+// Dequantize: the 16 units of 8 groups of the block go round-robin over the block's unit slots
+// (4 waves for float, 8 half-waves for half).
 template <typename T, int BITS>
-__device__ __forceinline__ void dequantize_wave32(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
-                                                  const T* __restrict__ mn, int64_t numel, int64_t N, int64_t wave,
-                                                  int lane, T* __restrict__ out) {
+__device__ __forceinline__ void dequantize_block128(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
+                                                    const T* __restrict__ mn, int64_t numel, int64_t N, int64_t lb,
+                                                    T* __restrict__ out) {
   constexpr int LPU = GROUP / Elem<T>::kDqWidth;  // lanes per unit
-  constexpr int UPW = 64 / LPU;                   // units a wave works on at a time
+  constexpr int SLOTS = 256 / LPU;
+  const int slot = threadIdx.x / LPU, l = threadIdx.x % LPU;
 #pragma unroll 1
-  for (int it = 0; it < 4 / UPW; it++) {
-    const int64_t unit = wave * 4 + it * UPW + lane / LPU;
-    if (unit * ROW_GROUPS < N) dequantize_8groups<T, BITS>(packed, scale, mn, numel, N, unit, lane % LPU, out);
+  for (int it = 0; it < 16 / SLOTS; it++) {
+    const int64_t unit = lb * 16 + it * SLOTS + slot;
+    if (unit * ROW_GROUPS < N) dequantize_8groups<T, BITS>(packed, scale, mn, numel, N, unit, l, out);
   }
 }
 
@@ -899,74 +902,46 @@ __device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ t
   return lo;
 }
 
-template <int NOISE>
+// One launch per width: blocks whose tensor has another width leave at once, so every width gets a
+// kernel with its own register allocation.
+template <int BITS, int NOISE>
 __global__ void __launch_bounds__(256)
 quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
-                        const int64_t* __restrict__ plan, uint8_t* __restrict__ packed_arena, uint8_t* __restrict__ scale_arena,
-                        uint8_t* __restrict__ min_arena) {
+                        const int64_t* __restrict__ plan, uint8_t* __restrict__ packed_arena,
+                        uint8_t* __restrict__ scale_arena, uint8_t* __restrict__ min_arena) {
   if (plan[1] == 0) return;  // the plan did not fit the arena or held an invalid width
   const int t = batch_find(table, L, blockIdx.x);
+  if (bits[t] != BITS) return;
   const gact_batch_entry ent = table[t];
-  const int bt = bits[t];
   const int64_t N = (ent.numel + GROUP - 1) / GROUP;
-  const int64_t row = ((int64_t)blockIdx.x - ent.first_block) * 16 + (threadIdx.x >> 4);
-  if (row * ROW_GROUPS >= N) return;
-  const int i = threadIdx.x & 15;
+  const int64_t lb = (int64_t)blockIdx.x - ent.first_block;
   uint8_t* packed = packed_arena + ent.packed_offset;
   uint8_t* sc = scale_arena + ent.stats_offset * 4;
   uint8_t* mn = min_arena + ent.stats_offset * 4;
-#define GACT_QB(T, B) \
-  quantize_row<T, B, NOISE, false>((const T*)ent.x, ent.numel, N, row, i, packed, (T*)sc, (T*)mn, (T*)nullptr, ent.seed, nullptr)
-  if (ent.dtype == GACT_F32) {
-    switch (bt) {
-      case 1: GACT_QB(float, 1); break;
-      case 2: GACT_QB(float, 2); break;
-      case 4: GACT_QB(float, 4); break;
-      case 8: GACT_QB(float, 8); break;
-    }
-  } else {
-    switch (bt) {
-      case 1: GACT_QB(f16, 1); break;
-      case 2: GACT_QB(f16, 2); break;
-      case 4: GACT_QB(f16, 4); break;
-      case 8: GACT_QB(f16, 8); break;
-    }
-  }
-#undef GACT_QB
+  if (ent.dtype == GACT_F32)
+    quantize_block128<float, BITS, NOISE>((const float*)ent.x, ent.numel, N, lb, packed, (float*)sc, (float*)mn, ent.seed);
+  else
+    quantize_block128<f16, BITS, NOISE>((const f16*)ent.x, ent.numel, N, lb, packed, (f16*)sc, (f16*)mn, ent.seed);
 }
 
+template <int BITS>
 __global__ void __launch_bounds__(256)
 dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
-                          const int64_t* __restrict__ plan, const uint8_t* __restrict__ packed_arena, const uint8_t* __restrict__ scale_arena,
-                          const uint8_t* __restrict__ min_arena) {
-  if (plan[1] == 0) return;  // the plan did not fit the arena or held an invalid width
+                          const int64_t* __restrict__ plan, const uint8_t* __restrict__ packed_arena,
+                          const uint8_t* __restrict__ scale_arena, const uint8_t* __restrict__ min_arena) {
+  if (plan[1] == 0) return;
   const int t = batch_find(table, L, blockIdx.x);
+  if (bits[t] != BITS) return;
   const gact_batch_entry ent = table[t];
-  const int bt = bits[t];
   const int64_t N = (ent.numel + GROUP - 1) / GROUP;
-  const int64_t wave = ((int64_t)blockIdx.x - ent.first_block) * 4 + (threadIdx.x >> 6);  // 32 groups per wave
-  if (wave * 32 >= N) return;
-  const int i = threadIdx.x & 63;
+  const int64_t lb = (int64_t)blockIdx.x - ent.first_block;
   const uint8_t* packed = packed_arena + ent.packed_offset;
   const uint8_t* sc = scale_arena + ent.stats_offset * 4;
   const uint8_t* mn = min_arena + ent.stats_offset * 4;
-#define GACT_DB(T, B) dequantize_wave32<T, B>(packed, (const T*)sc, (const T*)mn, ent.numel, N, wave, i, (T*)ent.x)
-  if (ent.dtype == GACT_F32) {
-    switch (bt) {
-      case 1: GACT_DB(float, 1); break;
-      case 2: GACT_DB(float, 2); break;
-      case 4: GACT_DB(float, 4); break;
-      case 8: GACT_DB(float, 8); break;
-    }
-  } else {
-    switch (bt) {
-      case 1: GACT_DB(f16, 1); break;
-      case 2: GACT_DB(f16, 2); break;
-      case 4: GACT_DB(f16, 4); break;
-      case 8: GACT_DB(f16, 8); break;
-    }
-  }
-#undef GACT_DB
+  if (ent.dtype == GACT_F32)
+    dequantize_block128<float, BITS>(packed, (const float*)sc, (const float*)mn, ent.numel, N, lb, (float*)ent.x);
+  else
+    dequantize_block128<f16, BITS>(packed, (const f16*)sc, (const f16*)mn, ent.numel, N, lb, (f16*)ent.x);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1270,17 +1245,18 @@ int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, in
   if (!aligned16(packed_arena)) return GACT_EALIGN;
   const dim3 grid((unsigned)total_blocks), block(256);
   hipStream_t s = (hipStream_t)stream;
+#define GACT_LAUNCH_QB(B, M)                                                                                  \
+  hipLaunchKernelGGL((quantize_batched_kernel<B, M>), grid, block, 0, s, table, bits, (int)L, plan,          \
+                     (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena)
+#define GACT_LAUNCH_QB_ALL(M) \
+  do { GACT_LAUNCH_QB(1, M); GACT_LAUNCH_QB(2, M); GACT_LAUNCH_QB(4, M); GACT_LAUNCH_QB(8, M); } while (0)
   switch (noise_mode) {
-    case GACT_NOISE_CONST:
-      hipLaunchKernelGGL((quantize_batched_kernel<GACT_NOISE_CONST>), grid, block, 0, s, table, bits, (int)L, plan, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena);
-      break;
-    case GACT_NOISE_REF:
-      hipLaunchKernelGGL((quantize_batched_kernel<GACT_NOISE_REF>), grid, block, 0, s, table, bits, (int)L, plan, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena);
-      break;
-    default:
-      hipLaunchKernelGGL((quantize_batched_kernel<GACT_NOISE_FAST>), grid, block, 0, s, table, bits, (int)L, plan, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena);
-      break;
+    case GACT_NOISE_CONST: GACT_LAUNCH_QB_ALL(GACT_NOISE_CONST); break;
+    case GACT_NOISE_REF: GACT_LAUNCH_QB_ALL(GACT_NOISE_REF); break;
+    default: GACT_LAUNCH_QB_ALL(GACT_NOISE_FAST); break;
   }
+#undef GACT_LAUNCH_QB_ALL
+#undef GACT_LAUNCH_QB
   return launch_status();
 }
 
@@ -1291,8 +1267,16 @@ int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, 
   if (L == 0 || total_blocks == 0) return GACT_OK;
   if (!table || !bits || !plan || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena)) return GACT_EALIGN;
-  hipLaunchKernelGGL(dequantize_batched_kernel, dim3((unsigned)total_blocks), dim3(256), 0, (hipStream_t)stream, table, bits, (int)L,
-                     plan, (const uint8_t*)packed_arena, (const uint8_t*)scale_arena, (const uint8_t*)min_arena);
+  const dim3 grid((unsigned)total_blocks), block(256);
+  hipStream_t s = (hipStream_t)stream;
+#define GACT_LAUNCH_DB(B)                                                                                    \
+  hipLaunchKernelGGL((dequantize_batched_kernel<B>), grid, block, 0, s, table, bits, (int)L, plan,           \
+                     (const uint8_t*)packed_arena, (const uint8_t*)scale_arena, (const uint8_t*)min_arena)
+  GACT_LAUNCH_DB(1);
+  GACT_LAUNCH_DB(2);
+  GACT_LAUNCH_DB(4);
+  GACT_LAUNCH_DB(8);
+#undef GACT_LAUNCH_DB
   return launch_status();
 }
 

@@ -111,8 +111,9 @@ typedef struct gact_batch_entry {
 int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t capacity, int64_t* plan,
                     void* stream);
 
-/* Quantize / dequantize all L tensors of the table in one grid of `total_blocks` blocks (the sum of
- * ceil(N_i/128)), each tensor at its own bits[i] read from device memory.  Scale and min of tensor i
+/* Quantize / dequantize all L tensors of the table over a grid of `total_blocks` blocks (the sum of
+ * ceil(N_i/128)), each tensor at its own bits[i] read from device memory; the grid is launched once per
+ * width (four launches, blocks of tensors at another width leave at once).  Scale and min of tensor i
  * are written at byte offset 4*stats_offset of their arenas.  Results equal a loop of gact_quantize /
  * gact_dequantize over the tensors (gact/gact/quantizer.py:95-142 drives the reference one tensor at a
  * time).  `plan` is the array gact_batch_plan filled. */
