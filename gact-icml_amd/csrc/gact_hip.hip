@@ -506,17 +506,17 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
 // groups are written, each store instruction covering whole groups contiguously.
 // quantization_cuda_kernel.cu:149-177.
 // ------------------------------------------------------------------------------------------------
-template <typename T, int BITS>
-__device__ __forceinline__ void dequantize_8groups(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
-                                                   const T* __restrict__ mn, int64_t numel, int64_t N, int64_t unit,
-                                                   int l, T* __restrict__ out) {
+template <typename T, int BITS, int SGS>
+__device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
+                                                const T* __restrict__ mn, int64_t numel, int64_t N, int64_t unit,
+                                                int l, T* __restrict__ out) {
   constexpr int WPT = 8 / BITS;
   constexpr int W = Elem<T>::kDqWidth;
-  const int64_t sg0 = unit * BITS;
+  const int64_t sg0 = unit * SGS;
   const int64_t n_sg = (N + WPT - 1) / WPT;
-  uint32_t w[BITS][W / 4];
+  uint32_t w[SGS][W / 4];
 #pragma unroll
-  for (int it = 0; it < BITS; it++) {
+  for (int it = 0; it < SGS; it++) {
     const uint8_t* p = packed + (sg0 + it) * GROUP + W * l;
     const bool live = sg0 + it < n_sg;
     if (W == 4) {
@@ -529,7 +529,7 @@ __device__ __forceinline__ void dequantize_8groups(const uint8_t* __restrict__ p
     }
   }
 #pragma unroll
-  for (int it = 0; it < BITS; it++) {
+  for (int it = 0; it < SGS; it++) {
 #pragma unroll
     for (int ni = 0; ni < WPT; ni++) {
       const int64_t n = (sg0 + it) * WPT + ni;
@@ -583,7 +583,7 @@ __device__ __forceinline__ void dequantize_block128(const uint8_t* __restrict__ 
 #pragma unroll 1
   for (int it = 0; it < 16 / SLOTS; it++) {
     const int64_t unit = lb * 16 + it * SLOTS + slot;
-    if (unit * ROW_GROUPS < N) dequantize_8groups<T, BITS>(packed, scale, mn, numel, N, unit, l, out);
+    if (unit * ROW_GROUPS < N) dequantize_unit<T, BITS, BITS>(packed, scale, mn, numel, N, unit, l, out);
   }
 }
 
@@ -611,6 +611,14 @@ __device__ __forceinline__ void minimax_row(const T* __restrict__ x, int64_t N, 
 // ------------------------------------------------------------------------------------------------
 // Single-tensor kernels.
 // ------------------------------------------------------------------------------------------------
+// groups a single-tensor dequantize unit (a wave for float, half a wave for half) covers
+#ifndef GACT_DQ_GROUPS
+#define GACT_DQ_GROUPS 8
+#endif
+__host__ __device__ constexpr int dq_supergroups(int bits) {
+  return GACT_DQ_GROUPS / (8 / bits) > 0 ? GACT_DQ_GROUPS / (8 / bits) : 1;
+}
+
 // One super-group per 16-lane row: short waves, many of them.
 template <typename T, int BITS, int NOISE, bool GIVEN>
 __global__ void __launch_bounds__(256)
@@ -628,8 +636,9 @@ dequantize_kernel(const uint8_t* __restrict__ packed, const T* __restrict__ scal
                   int64_t numel, int64_t N, T* __restrict__ out) {
   constexpr int LPU = GROUP / Elem<T>::kDqWidth;  // lanes per unit of 8 groups: 64 (float) or 32 (half)
   const int64_t unit = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / LPU;
-  if (unit * ROW_GROUPS >= N) return;
-  dequantize_8groups<T, BITS>(packed, scale, mn, numel, N, unit, threadIdx.x % LPU, out);
+  constexpr int SGS = dq_supergroups(BITS);
+  if (unit * (SGS * (8 / BITS)) >= N) return;
+  dequantize_unit<T, BITS, SGS>(packed, scale, mn, numel, N, unit, threadIdx.x % LPU, out);
 }
 
 template <typename T>
@@ -955,9 +964,17 @@ inline int launch_status() { return hipGetLastError() == hipSuccess ? GACT_OK : 
 
 // one 16-lane row per unit of work (a super-group for quantize / dequantize, 8 groups for minimax);
 // 16 rows per 256-thread block
-inline void row_grid(int64_t rows, dim3* grid, dim3* block) {
-  *grid = dim3((unsigned)((rows + 15) / 16));
-  *block = dim3(256);
+inline void row_grid(int64_t rows, dim3* grid, dim3* block, int threads = 256) {
+  const int rows_per_block = threads / 16;
+  *grid = dim3((unsigned)((rows + rows_per_block - 1) / rows_per_block));
+  *block = dim3(threads);
+}
+// Workgroup size of the quantize kernel.  A row's work grows with 8/bits groups; the long-running
+// low-width rows schedule better as single-wave workgroups (measured: float 2 bit 5.7 -> 6.2 TB/s,
+// 1 bit 5.4 -> 6.0 TB/s), the short high-width ones as four waves.
+inline int quantize_threads(int bits, size_t elem_size) {
+  const int wide_from = elem_size == 4 ? 8 : 4;
+  return bits >= wide_from ? 256 : 64;
 }
 inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8 / bits); }
 
@@ -965,7 +982,7 @@ template <typename T, int BITS, bool GIVEN>
 int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, T* scale, T* mn, T* mx, int noise_mode,
                     uint64_t seed, const float* noise, hipStream_t stream) {
   dim3 grid, block;
-  row_grid(supergroups(N, BITS), &grid, &block);
+  row_grid(supergroups(N, BITS), &grid, &block, quantize_threads(BITS, sizeof(T)));
   switch (noise_mode) {
     case GACT_NOISE_CONST:
       hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_CONST, GIVEN>), grid, block, 0, stream, x, numel, N,
@@ -1006,7 +1023,8 @@ int dispatch_dequantize(int bits, const uint8_t* packed, const T* scale, const T
                         hipStream_t stream) {
   // a unit of 8 groups takes 256 / (16 / sizeof(T)) lanes
   const int64_t units_per_block = 256 / (GROUP / (16 / (int64_t)sizeof(T)));
-  const dim3 grid((unsigned)(((N + ROW_GROUPS - 1) / ROW_GROUPS + units_per_block - 1) / units_per_block)), block(256);
+  const int64_t unit_groups = (int64_t)dq_supergroups(bits) * (8 / bits);
+  const dim3 grid((unsigned)(((N + unit_groups - 1) / unit_groups + units_per_block - 1) / units_per_block)), block(256);
   switch (bits) {
     case 1: hipLaunchKernelGGL((dequantize_kernel<T, 1>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
     case 2: hipLaunchKernelGGL((dequantize_kernel<T, 2>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
