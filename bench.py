@@ -188,6 +188,34 @@ def run_config5(torch, steps, warmup, seed=42):
     q_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / steps
     d_ms = sum(e[2].elapsed_time(e[3]) for e in ev) / steps
     wall_ms = (t1 - t0) * 1e3 / steps
+
+    # the same tensors and widths one call per tensor (what a hook-driven loop does), for comparison
+    singles = []
+    for x, o, b, sd in zip(xs, outs, host_bits, seeds):
+        N = (x.numel() + 255) // 256
+        singles.append((x, o, b, sd, torch.empty((lib.gact_packed_bytes(b, N, 1, 256) + 1,), dtype=torch.int8, device="cuda"),
+                        torch.empty((N,), dtype=x.dtype, device="cuda"), torch.empty((N,), dtype=x.dtype, device="cuda")))
+
+    def loop_q():
+        for x, o, b, sd, pk, s1, m1 in singles:
+            lib.gact_quantize(x.data_ptr(), 1, x.numel(), b, _abi.NOISE_FAST, sd, None, pk.data_ptr(), s1.data_ptr(),
+                              m1.data_ptr(), None, st)
+
+    def loop_d():
+        for x, o, b, sd, pk, s1, m1 in singles:
+            lib.gact_dequantize(pk.data_ptr(), b, s1.data_ptr(), m1.data_ptr(), 1, x.numel(), o.data_ptr(), st)
+
+    loop_ms = []
+    for fn in (loop_q, loop_d):
+        fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(5):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        loop_ms.append(e0.elapsed_time(e1) / 5)
     return {
         "workload": "config5", "desc": "120 fp16 Swin-Tiny-like tensors, widths by calc_precision on the GPU (budget "
                                        "2 bits/element), one batched mixed-width quantize + dequantize",
@@ -197,6 +225,9 @@ def run_config5(torch, steps, warmup, seed=42):
         "calc_precision": {"ms": a_ms},
         "quantize": {"ms": q_ms, "gbs": per_dir / (q_ms * 1e-3) / 1e9},
         "dequantize": {"ms": d_ms, "gbs": per_dir / (d_ms * 1e-3) / 1e9},
+        "tensor_by_tensor": {"quantize_ms": loop_ms[0], "dequantize_ms": loop_ms[1],
+                             "quantize_gbs": per_dir / (loop_ms[0] * 1e-3) / 1e9,
+                             "dequantize_gbs": per_dir / (loop_ms[1] * 1e-3) / 1e9},
     }
 
 

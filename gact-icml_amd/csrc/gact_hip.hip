@@ -828,27 +828,19 @@ __host__ __device__ inline float prec_key(float C, int b, int64_t w) {
 }
 __host__ __device__ inline bool prec_valid_bits(int b) { return b == 1 || b == 2 || b == 4 || b == 8 || b == 32; }
 
-#define PREC_MAX_L 4096
-__global__ void __launch_bounds__(64)
-calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, const int64_t* __restrict__ w,
-                      int L, double target, int32_t* __restrict__ status) {
-  __shared__ float key_s[PREC_MAX_L];
-  __shared__ int32_t b_s[PREC_MAX_L];
-  const int lane = threadIdx.x;
-  double part = 0.0;
-  for (int idx = lane; idx < L; idx += 64) {
-    const int bi = b[idx];
-    b_s[idx] = bi;
-    if (bi > 1) {
-      key_s[idx] = prec_key(C[idx], bi, w[idx]);
-      part += (double)((int64_t)bi * w[idx]);
-    }
-  }
-  // every term is an integer; the sum is exact (and order-free) below 2^53
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) part += __shfl_xor(part, off, 64);
-  double b_sum = part;
-  __syncthreads();
+#define PREC_MAX_L 4096      /* tensors the device kernel handles (LDS tables) */
+#define PREC_SORT_MAX_L 1024 /* tensors the sorting path handles (4 candidate steps each) */
+
+// The sequential restatement of the heap loop by one wave: each step is a 64-lane argmax.  Used when the
+// table is too long for the sorting path or a tensor's step keys do not decrease (never the case for the
+// non-negative sensitivities the callers produce).
+__device__ void calc_precision_sequential(int32_t* __restrict__ b_s, float* __restrict__ key_s,
+                                          const float* __restrict__ C, const int64_t* __restrict__ w, int L,
+                                          double b_sum, double target, int* rc_out) {
+  const int lane = threadIdx.x;  // threadIdx.x < 64
+  for (int idx = lane; idx < L; idx += 64)
+    if (b_s[idx] > 1) key_s[idx] = prec_key(C[idx], b_s[idx], w[idx]);
+  __builtin_amdgcn_wave_barrier();
   int rc = 0;
   while (b_sum > target) {
     float best_key = 0.0f;
@@ -869,16 +861,146 @@ calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, cons
     const int cur = b_s[best];
     const int nb = prec_next_bits(cur);
     const int64_t wb = w[best];
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();
     if (lane == 0) {
       b_s[best] = nb;
       if (nb > 1) key_s[best] = prec_key(C[best], nb, wb);
     }
     b_sum -= (double)(wb * (int64_t)(cur - nb));
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  *rc_out = rc;
+}
+
+// order-preserving map of a float key to an unsigned integer (+0 and -0 compare equal in the heap)
+__device__ __forceinline__ uint32_t sortable_key(float k) {
+  if (k == 0.0f) k = 0.0f;
+  const uint32_t u = __builtin_bit_cast(uint32_t, k);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// The greedy pops candidates (tensor i, step s) in descending (key, i) order.  A tensor's steps have
+// strictly decreasing keys, so that order is the descending sort of ALL candidate steps by
+// (key, index, earlier step first); the loop `while (b_sum > target) pop` then takes a prefix of it.
+// 256 threads: build up to 4 candidates per tensor, bitonic-sort them in LDS, prefix-sum the savings
+// (integers, exact in double), apply the prefix.  Falls back to the sequential loop when that order
+// argument does not hold.
+__global__ void __launch_bounds__(256)
+calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, const int64_t* __restrict__ w,
+                      int L, double target, int32_t* __restrict__ status) {
+  __shared__ uint64_t cand[4 * PREC_SORT_MAX_L];  // 32 KB; the sequential path reuses it for its float keys
+  __shared__ int32_t b_s[PREC_MAX_L];
+  __shared__ double part_s[256];
+  __shared__ int flag_s;
+  const int tid = threadIdx.x;
+  const bool sortable = L <= PREC_SORT_MAX_L;
+  int M = 4;
+  while (M < 4 * L) M <<= 1;
+  if (tid == 0) flag_s = 0;
+  if (sortable)
+    for (int t = tid; t < M; t += 256) cand[t] = 0;  // 0 sorts after every real candidate
+  __syncthreads();
+
+  double part = 0.0;
+  bool bad_order = false, bad_width = false;
+  for (int idx = tid; idx < L; idx += 256) {
+    const int bi = b[idx];
+    b_s[idx] = bi;
+    if (!prec_valid_bits(bi)) {
+      bad_width = true;
+    } else if (bi > 1) {
+      const int64_t wi = w[idx];
+      part += (double)((int64_t)bi * wi);
+      if (sortable) {
+        const float Ci = C[idx];
+        float prev = __builtin_inff();
+        int cur = bi, st = 0;
+        while (cur > 1 && st < 4) {
+          const float k = prec_key(Ci, cur, wi);
+          if (!(k < prev) && !(k == prev && k == 0.0f)) bad_order = true;  // also catches NaN
+          cand[idx * 4 + st] = ((uint64_t)sortable_key(k) << 32) | ((uint32_t)idx << 2) | (uint32_t)(3 - st);
+          prev = k;
+          cur = prec_next_bits(cur);
+          st++;
+        }
+        if (cur > 1) bad_order = true;  // a width the 4-step descent does not know
+      }
+    }
+  }
+  part_s[tid] = part;
+  if (bad_order) flag_s = 1;
+  __syncthreads();
+  if (bad_width) flag_s = 3;
+  __syncthreads();
+  if (flag_s == 3) {  // a width outside {1,2,4,8,32}: leave b as it is
+    if (status && tid == 0) *status = GACT_EINVAL;
+    return;
+  }
+  // every term is an integer; the sum is exact (and order-free) below 2^53
+  for (int off = 128; off >= 1; off >>= 1) {
+    if (tid < off) part_s[tid] += part_s[tid + off];
     __syncthreads();
   }
-  for (int idx = lane; idx < L; idx += 64) b[idx] = b_s[idx];
-  if (status && lane == 0) *status = rc;
+  const double b_sum0 = part_s[0];
+  const bool sequential = !sortable || flag_s != 0;
+  __syncthreads();
+
+  int rc = 0;
+  if (sequential) {
+    if (tid < 64) calc_precision_sequential(b_s, reinterpret_cast<float*>(cand), C, w, L, b_sum0, target, &rc);
+  } else {
+    // bitonic sort, descending
+    for (int k = 2; k <= M; k <<= 1) {
+      for (int j = k >> 1; j > 0; j >>= 1) {
+        for (int t = tid; t < M; t += 256) {
+          const int o = t ^ j;
+          if (o > t) {
+            const uint64_t x = cand[t], y = cand[o];
+            const bool descending = (t & k) == 0;
+            if (descending ? x < y : x > y) { cand[t] = y; cand[o] = x; }
+          }
+        }
+        __syncthreads();
+      }
+    }
+    // savings of the sorted candidates, chunked over the threads
+    const int per = M / 256 > 0 ? M / 256 : 1;
+    const int lo = tid * per, hi = lo + per < M ? lo + per : M;
+    double mine = 0.0;
+    for (int t = lo; t < hi && t < M; t++) {
+      const uint64_t c = cand[t];
+      if (c == 0) break;
+      const int idx = (int)((uint32_t)c >> 2), st = 3 - (int)(c & 3u);
+      int cur = b[idx];
+      for (int q = 0; q < st; q++) cur = prec_next_bits(cur);
+      mine += (double)(w[idx] * (int64_t)(cur - prec_next_bits(cur)));
+    }
+    part_s[tid] = (lo < M) ? mine : 0.0;
+    __syncthreads();
+    if (tid == 0) {  // exclusive prefix over 256 partial sums
+      double run = 0.0;
+      for (int t = 0; t < 256; t++) { const double v = part_s[t]; part_s[t] = run; run += v; }
+      if (b_sum0 - run > target) flag_s = 2;  // every step taken and still over budget
+    }
+    __syncthreads();
+    double running = b_sum0 - part_s[tid];
+    for (int t = lo; t < hi && t < M; t++) {
+      const uint64_t c = cand[t];
+      if (c == 0 || !(running > target)) break;
+      const int idx = (int)((uint32_t)c >> 2), st = 3 - (int)(c & 3u);
+      int cur = b[idx];
+      for (int q = 0; q < st; q++) cur = prec_next_bits(cur);
+      const int nb = prec_next_bits(cur);
+      atomicMin(&b_s[idx], nb);
+      running -= (double)(w[idx] * (int64_t)(cur - nb));
+    }
+    __syncthreads();
+    if (flag_s == 2) rc = GACT_EBUDGET;
+  }
+  __syncthreads();
+  for (int idx = tid; idx < L; idx += 256) b[idx] = b_s[idx];
+  if (status && tid == 0) *status = rc;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1239,7 +1361,7 @@ int gact_calc_precision_device(int32_t* b, const float* C, const int64_t* w, int
   if (L > PREC_MAX_L) return GACT_ESHAPE;
   if (L == 0) return GACT_OK;
   if (!b || !C || !w) return GACT_EINVAL;
-  hipLaunchKernelGGL(calc_precision_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, b, C, w, (int)L, target, status);
+  hipLaunchKernelGGL(calc_precision_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, b, C, w, (int)L, target, status);
   return launch_status();
 }
 

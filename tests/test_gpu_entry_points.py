@@ -116,6 +116,42 @@ def test_calc_precision_device_matches_host_and_oracle(L, init, avg):
     assert status.item() == 0
 
 
+def test_calc_precision_device_adversarial_orders():
+    # ties, near ties, zero and infinite sensitivities (the last two leave the sorting path), long tables
+    rng = np.random.default_rng(77)
+    cases = []
+    for t in range(40):
+        L = int(rng.integers(1, 300))
+        base = np.float32(np.exp(rng.normal(0, 1)))
+        C = (np.full(L, base, np.float32).view(np.int32) + rng.integers(-2, 3, L).astype(np.int32)).view(np.float32)
+        w = np.full(L, int(rng.choice([256, 4096, 65536])), np.int64)
+        cases.append((C, w, int(rng.choice([8, 32])), float(rng.choice([1.0, 1.5, 2.0, 3.0, 5.0]))))
+    cases.append((np.zeros(50, np.float32), np.full(50, 1024, np.int64), 8, 2.0))
+    cases.append((np.array([0.0, 1.0, 0.0, 2.0, 0.0], np.float32), np.full(5, 512, np.int64), 32, 2.0))
+    cases.append((np.array([np.inf, 1.0, np.inf, 2.0], np.float32), np.full(4, 512, np.int64), 8, 2.0))
+    big = 1500                                       # beyond the sorting path: the sequential path
+    cases.append((np.exp(rng.normal(0, 2, big)).astype(np.float32), (rng.integers(1, 50, big) * 256).astype(np.int64), 8, 2.0))
+    cases.append((np.exp(rng.normal(0, 2, 1024)).astype(np.float32), (rng.integers(1, 50, 1024) * 256).astype(np.int64), 32, 3.0))
+    for C, w, init, avg in cases:
+        L = C.size
+        target = avg * float(w.sum())
+        want = oracle.calc_precision(np.full(L, init, np.int32), C, w, target)
+        status = torch.full((1,), 99, dtype=torch.int32, device="cuda")
+        dev = ext_calc_precision.calc_precision_device(torch.full((L,), init, dtype=torch.int32, device="cuda"),
+                                                       torch.from_numpy(C).cuda(), torch.from_numpy(w).cuda(), target,
+                                                       status)
+        np.testing.assert_array_equal(dev.cpu().numpy(), want)
+        assert status.item() == 0
+
+
+def test_calc_precision_device_rejects_unknown_widths():
+    b = torch.tensor([8, 3, 8], dtype=torch.int32, device="cuda")
+    status = torch.zeros((1,), dtype=torch.int32, device="cuda")
+    ext_calc_precision.calc_precision_device(b, torch.ones(3, device="cuda"),
+                                             torch.full((3,), 256, dtype=torch.int64, device="cuda"), 100.0, status)
+    assert status.item() == -1 and b.cpu().tolist() == [8, 3, 8]
+
+
 def test_calc_precision_device_reports_unreachable_budget():
     L = 5
     b = torch.full((L,), 8, dtype=torch.int32, device="cuda")
