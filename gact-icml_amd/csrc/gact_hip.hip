@@ -171,6 +171,13 @@ template <> struct Elem<float> {
         hi = __builtin_fmaxf(hi, st.v[k][e]);
       }
   }
+  // min and max of the whole group, in every lane of the row
+  __device__ static __forceinline__ void group_minmax(const Store& st, float& lo_out, float& hi_out) {
+    float lo = init_lo(), hi = init_hi();
+    minmax(st, lo, hi);
+    lo_out = row_all_min(lo);
+    hi_out = row_all_max(hi);
+  }
   __device__ static __forceinline__ void store_codes(uint8_t* p, const uint32_t (&b)[4]) {
     // the reference accumulates in a uint8_t: keep the low 8 bits of every byte
     uint32_t w = (b[0] & 0xffu) | ((b[1] & 0xffu) << 8) | ((b[2] & 0xffu) << 16) | (b[3] << 24);
@@ -250,6 +257,38 @@ template <> struct Elem<f16> {
       }
     lo = __builtin_fminf((float)l.x, (float)l.y);
     hi = __builtin_fmaxf((float)h.x, (float)h.y);
+  }
+  // min and max of the whole group, in every lane of the row: packed per-lane min / max, then ONE row
+  // reduction over the pair {min, -max} with packed min
+  __device__ static __forceinline__ void group_minmax(const Store& st, f16& lo_out, f16& hi_out) {
+    f16x2 l = st.v[0][0], h = st.v[0][0];
+#pragma unroll
+    for (int k = 0; k < 2; k++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        if (k + j == 0) continue;
+        l = __builtin_elementwise_min(l, st.v[k][j]);
+        h = __builtin_elementwise_max(h, st.v[k][j]);
+      }
+    // NaN elements never win a min / max; start values +-inf only matter for an all-NaN group
+    const f16 inf = (f16)__builtin_inff();
+    const f16 lmin = __builtin_elementwise_min(__builtin_elementwise_min((f16)l.x, (f16)l.y), inf);
+    const f16 hmax = __builtin_elementwise_max(__builtin_elementwise_max((f16)h.x, (f16)h.y), (f16)-inf);
+    f16x2 m = {lmin, (f16)-hmax};
+#pragma unroll
+    for (int step = 8; step >= 1; step >>= 1) {
+      const int bits = __builtin_bit_cast(int, m);
+      int other;
+      switch (step) {
+        case 8: other = __builtin_amdgcn_update_dpp(bits, bits, DPP_ROW_ROR(8), 0xf, 0xf, false); break;
+        case 4: other = __builtin_amdgcn_update_dpp(bits, bits, DPP_ROW_ROR(4), 0xf, 0xf, false); break;
+        case 2: other = __builtin_amdgcn_update_dpp(bits, bits, DPP_ROW_ROR(2), 0xf, 0xf, false); break;
+        default: other = __builtin_amdgcn_update_dpp(bits, bits, DPP_ROW_ROR(1), 0xf, 0xf, false); break;
+      }
+      m = __builtin_elementwise_min(m, __builtin_bit_cast(f16x2, other));
+    }
+    lo_out = m.x;
+    hi_out = -m.y;
   }
   // range is a half operation; the quotient is a double narrowed to float and then to half
   __device__ static __forceinline__ f16 make_scale(f16 lo, f16 hi, int qmax) {
@@ -342,6 +381,18 @@ __device__ __forceinline__ void load_group(const T* __restrict__ x, int64_t nume
   }
 }
 
+// value of lane LANE of the row, in every lane of the row (DPP row_newbcast)
+template <int LANE>
+__device__ __forceinline__ uint32_t row_bcast_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x150 + LANE, 0xf, 0xf, false);
+}
+template <int LANE> __device__ __forceinline__ float row_bcast(float v) {
+  return __builtin_bit_cast(float, row_bcast_u32<LANE>(__builtin_bit_cast(uint32_t, v)));
+}
+template <int LANE> __device__ __forceinline__ f16 row_bcast(f16 v) {
+  return __builtin_bit_cast(f16, (uint16_t)row_bcast_u32<LANE>((uint32_t)__builtin_bit_cast(uint16_t, v)));
+}
+
 // 16-bit piece e of a pair of Philox words -> uniform of the fast stream
 __device__ __forceinline__ float fast_piece(uint32_t w0, uint32_t w1, int e) {
   const uint32_t w = (e & 2) ? w1 : w0;
@@ -408,7 +459,7 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
   const int64_t n0 = sg * WPT;
 
   typename Elem<T>::Store v[WPT];
-  T lo_t[WPT], s_t[WPT];
+  T lo_t[WPT], hi_t[WPT], s_t[WPT];
 #pragma unroll
   for (int ni = 0; ni < WPT; ni++) {
     if (n0 + ni < N) load_group<T>(x, numel, n0 + ni, i, v[ni]);
@@ -416,28 +467,43 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
 #pragma unroll
   for (int ni = 0; ni < WPT; ni++) {
     const int64_t n = n0 + ni;
+    lo_t[ni] = (T)0;
+    hi_t[ni] = (T)0;
     if (n < N) {
-      T lo_v, hi_v;
       if (GIVEN) {
-        lo_v = mn_io[n];
-        hi_v = mx_io[n];
+        lo_t[ni] = mn_io[n];
+        hi_t[ni] = mx_io[n];
       } else {
-        float lo = Elem<T>::init_lo(), hi = Elem<T>::init_hi();
-        Elem<T>::minmax(v[ni], lo, hi);
-        lo = row_all_min(lo);
-        hi = row_all_max(hi);
-        lo_v = Elem<T>::from_float(lo);
-        hi_v = Elem<T>::from_float(hi);
+        Elem<T>::group_minmax(v[ni], lo_t[ni], hi_t[ni]);
       }
-      T s = Elem<T>::make_scale(lo_v, hi_v, QMAX);
-      lo_t[ni] = lo_v;
-      s_t[ni] = s;
-      if (i == ni) {
-        scale_out[n] = s;
-        if (!GIVEN) {
-          mn_io[n] = lo_v;
-          if (mx_io) mx_io[n] = hi_v;
-        }
+    }
+  }
+  // one scale division per lane: lane j of the row takes group j % WPT, then the row shares the results
+  {
+    const int mine = i & (WPT - 1);
+    T lo_m = lo_t[0], hi_m = hi_t[0];
+#pragma unroll
+    for (int ni = 1; ni < WPT; ni++) {
+      lo_m = (mine == ni) ? lo_t[ni] : lo_m;
+      hi_m = (mine == ni) ? hi_t[ni] : hi_m;
+    }
+    const T s_m = Elem<T>::make_scale(lo_m, hi_m, QMAX);
+    if (i < WPT && n0 + i < N) {
+      scale_out[n0 + i] = s_m;
+      if (!GIVEN) {
+        mn_io[n0 + i] = lo_m;
+        if (mx_io) mx_io[n0 + i] = hi_m;
+      }
+    }
+    if (WPT == 1) {
+      s_t[0] = s_m;
+    } else {
+      s_t[0] = row_bcast<0>(s_m);
+      if (WPT > 1) s_t[1 % WPT] = row_bcast<1>(s_m);
+      if (WPT > 2) { s_t[2 % WPT] = row_bcast<2>(s_m); s_t[3 % WPT] = row_bcast<3>(s_m); }
+      if (WPT > 4) {
+        s_t[4 % WPT] = row_bcast<4>(s_m); s_t[5 % WPT] = row_bcast<5>(s_m);
+        s_t[6 % WPT] = row_bcast<6>(s_m); s_t[7 % WPT] = row_bcast<7>(s_m);
       }
     }
   }
@@ -597,13 +663,11 @@ __device__ __forceinline__ void minimax_row(const T* __restrict__ x, int64_t N, 
     if (n >= N) break;
     typename Elem<T>::Store v;
     load_group<T>(x, N * GROUP, n, i, v);
-    float lo = Elem<T>::init_lo(), hi = Elem<T>::init_hi();
-    Elem<T>::minmax(v, lo, hi);
-    lo = row_all_min(lo);
-    hi = row_all_max(hi);
+    T lo, hi;
+    Elem<T>::group_minmax(v, lo, hi);
     if (i == 0) {
-      mn[n] = Elem<T>::from_float(lo);
-      mx[n] = Elem<T>::from_float(hi);
+      mn[n] = lo;
+      mx[n] = hi;
     }
   }
 }
