@@ -594,13 +594,38 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
       w[it][W / 4 - 1] = t.y;
     }
   }
+  // scale and min of the unit's groups: 16-byte loads when the whole unit exists and the arrays allow it
+  constexpr int G = SGS * WPT;
+  constexpr int PER16 = 16 / (int)sizeof(T);
+  const int64_t g0 = sg0 * WPT;
+  T sv[G], mv[G];
+  if (G % PER16 == 0 && g0 + G <= N &&
+      ((reinterpret_cast<uintptr_t>(scale + g0) | reinterpret_cast<uintptr_t>(mn + g0)) & 15u) == 0) {
+    typedef T vec16 __attribute__((ext_vector_type(PER16)));
+#pragma unroll
+    for (int c = 0; c < G / PER16; c++) {
+      const vec16 a = *reinterpret_cast<const vec16*>(scale + g0 + c * PER16);
+      const vec16 m = *reinterpret_cast<const vec16*>(mn + g0 + c * PER16);
+#pragma unroll
+      for (int e = 0; e < PER16; e++) {
+        sv[c * PER16 + e] = a[e];
+        mv[c * PER16 + e] = m[e];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+      sv[g] = g0 + g < N ? scale[g0 + g] : (T)1;
+      mv[g] = g0 + g < N ? mn[g0 + g] : (T)0;
+    }
+  }
 #pragma unroll
   for (int it = 0; it < SGS; it++) {
 #pragma unroll
     for (int ni = 0; ni < WPT; ni++) {
       const int64_t n = (sg0 + it) * WPT + ni;
       if (n < N) {
-        const typename Elem<T>::Dq d = Elem<T>::dq_prepare(scale[n], mn[n]);
+        const typename Elem<T>::Dq d = Elem<T>::dq_prepare(sv[it * WPT + ni], mv[it * WPT + ni]);
         T v[W];
 #pragma unroll
         for (int e = 0; e < W; e++) {

@@ -68,7 +68,7 @@ class BatchedQuantizer:
             self.first_blocks.append(blocks)
             self.stats_offsets.append(groups)
             blocks += (N + GROUPS_PER_BLOCK - 1) // GROUPS_PER_BLOCK
-            groups += N
+            groups += (N + 7) // 8 * 8   # 32-byte aligned rows: the dequantize kernel reads them 16 bytes at a time
         self.total_blocks = blocks
         self.total_groups = groups
 
