@@ -184,3 +184,65 @@ def test_32bit_passthrough():
     assert torch.equal(q_min.reshape(-1), torch.min(x, dim=1).values)
     assert torch.equal(q_scale.reshape(-1), torch.max(x, dim=1).values - torch.min(x, dim=1).values)
     assert torch.equal(ops.op_dequantize(q, x.shape), x)
+
+
+def test_empty_tensor():
+    x = torch.empty((0, 256), device="cuda")
+    q = ops.op_quantize(x, 4, 0)
+    assert q[0].numel() == 1 and q[2].shape == (0, 1, 1) and q[3].shape == (0, 1, 1)
+    assert ops.op_dequantize(q, x.shape).shape == (0, 256)
+
+
+@pytest.mark.parametrize("bits", [1, 8])
+def test_more_than_2_to_31_elements(bits):
+    # indices beyond 32 bits: element offsets, byte offsets and Philox block numbers are 64-bit
+    numel = (1 << 31) + 256 * 24 + 100
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.empty(numel, dtype=torch.float16, device="cuda")
+    x.normal_(generator=g)
+    q = ops.op_quantize(x, bits, 9, rng_stream="deterministic")
+    out = ops.op_dequantize(q, x.shape)
+    torch.cuda.synchronize()
+    N = (numel + 255) // 256
+    wpt = 8 // bits
+    # oracle on the first and the last 4096 groups (whole byte rows, so the slices are self-contained)
+    for g0 in (0, (N - 4096) // 8 * 8):
+        g1 = min(g0 + 4096, N)
+        xs = x[g0 * 256: min(g1 * 256, numel)].cpu().numpy()
+        ref = oracle.op_quantize(xs, bits, oracle.NOISE_CONST)
+        nb = ref[0].size
+        b0 = (g0 // wpt) * 256
+        got = q[0][b0: b0 + nb].cpu().numpy().view(np.uint8)
+        assert np.array_equal(got, ref[0])
+        assert np.array_equal(q[2][g0:g1].cpu().numpy(), ref[2]) and np.array_equal(q[3][g0:g1].cpu().numpy(), ref[3])
+        want = oracle.op_dequantize(ref, xs.shape)
+        assert np.array_equal(out[g0 * 256: g0 * 256 + xs.size].cpu().numpy(), want)
+    # and the fast stream reaches the far end too: block numbers differ from their 32-bit truncation
+    qf = ops.op_quantize(x, bits, 9, rng_stream="fast")
+    g0 = (N - 4096) // 8 * 8
+    tail = x[g0 * 256:].cpu().numpy()
+    Nt = (tail.size + 255) // 256
+    # the oracle numbers elements from 0, so feed it the absolute indices through an injected noise tensor
+    idx = (np.arange(Nt * 256, dtype=np.uint64) + np.uint64(g0 * 256))
+    blk = idx >> np.uint64(3)
+    uu = np.empty(Nt * 256, np.float32)
+    cache = {}
+    for b in np.unique(blk[:: 8])[:64]:                 # 64 blocks = 512 elements are enough to pin the indexing
+        cache[int(b)] = oracle.philox4x32_10([0, 0, int(b) & 0xFFFFFFFF, int(b) >> 32], [9, 0])
+    sel = np.nonzero(np.isin(blk, np.array(list(cache), dtype=np.uint64)))[0]
+    for e in sel:
+        w = int(cache[int(blk[e])][(int(idx[e]) % 8) // 2])
+        h = (w >> 16) if (int(idx[e]) % 2) else (w & 0xFFFF)
+        uu[e] = (h + 0.5) / 65536.0
+    first = int(sel.max()) + 1                          # the selected elements are the first 512 of the tail
+    assert first == 512
+    ref = oracle.op_quantize(tail[:512], bits, oracle.NOISE_INJECT, 0, uu[:512])
+    # 512 elements = 2 groups; compare their codes field by field
+    pk = qf[0].cpu().numpy().view(np.uint8)
+    for n_local in range(2):
+        n = g0 + n_local
+        row, ni = divmod(n, wpt)
+        got = (pk[row * 256: row * 256 + 256] >> (ni * bits)) & (2 ** bits - 1)
+        rrow, rni = divmod(n_local, wpt)
+        want = (ref[0][rrow * 256: rrow * 256 + 256] >> (rni * bits)) & (2 ** bits - 1)
+        assert np.array_equal(got, want)
