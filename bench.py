@@ -151,7 +151,7 @@ def run_config5(torch, steps, warmup, seed=42):
     packed = torch.empty((bq.arena_bytes_for_budget(target),), dtype=torch.uint8, device="cuda")
     sc = torch.empty((bq.total_groups * 4,), dtype=torch.uint8, device="cuda")
     mn = torch.empty((bq.total_groups * 4,), dtype=torch.uint8, device="cuda")
-    plan = torch.empty((2,), dtype=torch.int64, device="cuda")
+    plan = torch.empty((6,), dtype=torch.int64, device="cuda")
     st = torch.cuda.current_stream().cuda_stream
 
     def allocate():
@@ -162,12 +162,14 @@ def run_config5(torch, steps, warmup, seed=42):
     def quantize():
         _abi.check(lib.gact_batch_plan(table_q.data_ptr(), bits.data_ptr(), L, packed.numel(), plan.data_ptr(), st))
         _abi.check(lib.gact_quantize_batched(table_q.data_ptr(), bits.data_ptr(), L, bq.total_blocks, _abi.NOISE_FAST,
-                                             plan.data_ptr(), packed.data_ptr(), sc.data_ptr(), mn.data_ptr(), st))
+                                             plan.data_ptr(), bq.block_map.data_ptr(), packed.data_ptr(), sc.data_ptr(),
+                                             mn.data_ptr(), st))
 
     def dequantize():
         _abi.check(lib.gact_batch_plan(table_d.data_ptr(), bits.data_ptr(), L, packed.numel(), plan.data_ptr(), st))
         _abi.check(lib.gact_dequantize_batched(table_d.data_ptr(), bits.data_ptr(), L, bq.total_blocks,
-                                               plan.data_ptr(), packed.data_ptr(), sc.data_ptr(), mn.data_ptr(), st))
+                                               plan.data_ptr(), bq.block_map.data_ptr(), packed.data_ptr(),
+                                               sc.data_ptr(), mn.data_ptr(), st))
 
     for _ in range(warmup):
         allocate(); quantize(); dequantize()

@@ -1095,22 +1095,49 @@ calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, cons
 // ------------------------------------------------------------------------------------------------
 // Batched launch over a table of tensors with device-resident bits.
 // ------------------------------------------------------------------------------------------------
-__global__ void batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int L,
-                                  int64_t capacity, int64_t* plan) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
-  int64_t off = 0;
-  bool ok = true;
-  for (int t = 0; t < L; t++) {
-    int bt = bits[t];
-    if (!(bt == 1 || bt == 2 || bt == 4 || bt == 8)) { ok = false; bt = 8; }
-    const int wpt = 8 / bt;
-    const int64_t N = (table[t].numel + GROUP - 1) / GROUP;
-    const int64_t n_round = (N + wpt - 1) / wpt * wpt;
-    table[t].packed_offset = off;
-    off += ((int64_t)bt * n_round * (GROUP / 8) + 255) / 256 * 256;
+// One wave: lane l sizes tensors l, l+64, ...; a running offset is carried across rounds of 64 with a
+// wave-wide inclusive scan.  plan[0] = arena bytes needed, plan[1] = ok flag, plan[2 + k] = number of
+// tensors at width 1 << k (the work kernels of a width nobody uses leave at once).
+__global__ void __launch_bounds__(64)
+batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int L, int64_t capacity,
+                  int64_t* plan) {
+  const int lane = threadIdx.x;
+  int64_t base = 0;
+  int bad = 0;
+  int cnt[4] = {0, 0, 0, 0};
+  for (int t0 = 0; t0 < L; t0 += 64) {
+    const int t = t0 + lane;
+    int64_t bytes = 0;
+    if (t < L) {
+      int bt = bits[t];
+      if (!(bt == 1 || bt == 2 || bt == 4 || bt == 8)) { bad = 1; bt = 8; }
+      cnt[bt == 1 ? 0 : bt == 2 ? 1 : bt == 4 ? 2 : 3]++;
+      const int wpt = 8 / bt;
+      const int64_t N = (table[t].numel + GROUP - 1) / GROUP;
+      const int64_t n_round = (N + wpt - 1) / wpt * wpt;
+      bytes = ((int64_t)bt * n_round * (GROUP / 8) + 255) / 256 * 256;
+    }
+    int64_t incl = bytes;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int64_t up = __shfl_up(incl, off, 64);
+      if (lane >= off) incl += up;
+    }
+    if (t < L) table[t].packed_offset = base + incl - bytes;
+    base += __shfl(incl, 63, 64);
   }
-  plan[0] = off;
-  plan[1] = (ok && off <= capacity) ? 1 : 0;
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    bad |= __shfl_xor(bad, off, 64);
+#pragma unroll
+    for (int k = 0; k < 4; k++) cnt[k] += __shfl_xor(cnt[k], off, 64);
+  }
+  if (lane == 0) {
+    plan[0] = base;
+    plan[1] = (!bad && base <= capacity) ? 1 : 0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) plan[2 + k] = cnt[k];
+  }
 }
 
 __device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ table, int L, int64_t block) {
@@ -1127,10 +1154,12 @@ __device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ t
 template <int BITS, int NOISE>
 __global__ void __launch_bounds__(256)
 quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
-                        const int64_t* __restrict__ plan, uint8_t* __restrict__ packed_arena,
-                        uint8_t* __restrict__ scale_arena, uint8_t* __restrict__ min_arena) {
-  if (plan[1] == 0) return;  // the plan did not fit the arena or held an invalid width
-  const int t = batch_find(table, L, blockIdx.x);
+                        const int64_t* __restrict__ plan, const int32_t* __restrict__ block_map,
+                        uint8_t* __restrict__ packed_arena, uint8_t* __restrict__ scale_arena,
+                        uint8_t* __restrict__ min_arena) {
+  // the plan did not fit the arena or held an invalid width, or no tensor has this width
+  if (plan[1] == 0 || plan[2 + (BITS == 1 ? 0 : BITS == 2 ? 1 : BITS == 4 ? 2 : 3)] == 0) return;
+  const int t = block_map ? block_map[blockIdx.x] : batch_find(table, L, blockIdx.x);
   if (bits[t] != BITS) return;
   const gact_batch_entry ent = table[t];
   const int64_t N = (ent.numel + GROUP - 1) / GROUP;
@@ -1147,10 +1176,11 @@ quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_
 template <int BITS>
 __global__ void __launch_bounds__(256)
 dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
-                          const int64_t* __restrict__ plan, const uint8_t* __restrict__ packed_arena,
-                          const uint8_t* __restrict__ scale_arena, const uint8_t* __restrict__ min_arena) {
-  if (plan[1] == 0) return;
-  const int t = batch_find(table, L, blockIdx.x);
+                          const int64_t* __restrict__ plan, const int32_t* __restrict__ block_map,
+                          const uint8_t* __restrict__ packed_arena, const uint8_t* __restrict__ scale_arena,
+                          const uint8_t* __restrict__ min_arena) {
+  if (plan[1] == 0 || plan[2 + (BITS == 1 ? 0 : BITS == 2 ? 1 : BITS == 4 ? 2 : 3)] == 0) return;
+  const int t = block_map ? block_map[blockIdx.x] : batch_find(table, L, blockIdx.x);
   if (bits[t] != BITS) return;
   const gact_batch_entry ent = table[t];
   const int64_t N = (ent.numel + GROUP - 1) / GROUP;
@@ -1464,8 +1494,8 @@ int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int
 }
 
 int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
-                          int noise_mode, const int64_t* plan, void* packed_arena, void* scale_arena, void* min_arena,
-                          void* stream) {
+                          int noise_mode, const int64_t* plan, const int32_t* block_map, void* packed_arena,
+                          void* scale_arena, void* min_arena, void* stream) {
   if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x7fffffffLL) return GACT_EINVAL;
   if (noise_mode != GACT_NOISE_CONST && noise_mode != GACT_NOISE_REF && noise_mode != GACT_NOISE_FAST)
     return GACT_EINVAL;  // injected noise is a single-tensor test mode
@@ -1476,7 +1506,7 @@ int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, in
   hipStream_t s = (hipStream_t)stream;
 #define GACT_LAUNCH_QB(B, M)                                                                                  \
   hipLaunchKernelGGL((quantize_batched_kernel<B, M>), grid, block, 0, s, table, bits, (int)L, plan,          \
-                     (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena)
+                     block_map, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena)
 #define GACT_LAUNCH_QB_ALL(M) \
   do { GACT_LAUNCH_QB(1, M); GACT_LAUNCH_QB(2, M); GACT_LAUNCH_QB(4, M); GACT_LAUNCH_QB(8, M); } while (0)
   switch (noise_mode) {
@@ -1490,8 +1520,8 @@ int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, in
 }
 
 int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
-                            const int64_t* plan, const void* packed_arena, const void* scale_arena,
-                            const void* min_arena, void* stream) {
+                            const int64_t* plan, const int32_t* block_map, const void* packed_arena,
+                            const void* scale_arena, const void* min_arena, void* stream) {
   if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x7fffffffLL) return GACT_EINVAL;
   if (L == 0 || total_blocks == 0) return GACT_OK;
   if (!table || !bits || !plan || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
@@ -1500,7 +1530,8 @@ int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, 
   hipStream_t s = (hipStream_t)stream;
 #define GACT_LAUNCH_DB(B)                                                                                    \
   hipLaunchKernelGGL((dequantize_batched_kernel<B>), grid, block, 0, s, table, bits, (int)L, plan,           \
-                     (const uint8_t*)packed_arena, (const uint8_t*)scale_arena, (const uint8_t*)min_arena)
+                     block_map, (const uint8_t*)packed_arena, (const uint8_t*)scale_arena,                 \
+                     (const uint8_t*)min_arena)
   GACT_LAUNCH_DB(1);
   GACT_LAUNCH_DB(2);
   GACT_LAUNCH_DB(4);

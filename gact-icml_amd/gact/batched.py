@@ -30,8 +30,8 @@ class BatchedPacked:
 
     def ok(self):
         """Synchronising check that the plan fitted the arena and every width was valid."""
-        need, ok = self.plan.tolist()
-        return bool(ok), need
+        vals = self.plan.tolist()
+        return bool(vals[1]), vals[0]
 
     def per_tensor(self, i):
         """Views (packed bytes, bits, scale[N,1,1], min[N,1,1]) of tensor i in op_quantize's format.
@@ -71,6 +71,12 @@ class BatchedQuantizer:
             groups += (N + 7) // 8 * 8   # 32-byte aligned rows: the dequantize kernel reads them 16 bytes at a time
         self.total_blocks = blocks
         self.total_groups = groups
+        # block -> tensor, fixed by the geometry: lets a block find its tensor with one load
+        bm = torch.empty((max(blocks, 1),), dtype=torch.int32)
+        for i in range(self.L):
+            end = self.first_blocks[i + 1] if i + 1 < self.L else blocks
+            bm[self.first_blocks[i]:end] = i
+        self.block_map = bm.to(self.device)
 
     # ---- arena sizing (host-side bounds; the exact need is computed on the device) ----
     def arena_bytes_for_budget(self, target_bits):
@@ -119,13 +125,13 @@ class BatchedQuantizer:
             packed = torch.empty((int(arena_bytes),), dtype=torch.uint8, device=self.device)
             scale = torch.empty((self.total_groups * 4,), dtype=torch.uint8, device=self.device)
             mn = torch.empty((self.total_groups * 4,), dtype=torch.uint8, device=self.device)
-            plan = torch.empty((2,), dtype=torch.int64, device=self.device)
+            plan = torch.empty((6,), dtype=torch.int64, device=self.device)
             st = torch.cuda.current_stream(self.device).cuda_stream
             _abi.check(lib.gact_batch_plan(table.data_ptr(), bits.data_ptr(), self.L, packed.numel(),
                                            plan.data_ptr(), st))
             _abi.check(lib.gact_quantize_batched(table.data_ptr(), bits.data_ptr(), self.L, self.total_blocks, mode,
-                                                 plan.data_ptr(), packed.data_ptr(), scale.data_ptr(),
-                                                 mn.data_ptr(), st))
+                                                 plan.data_ptr(), self.block_map.data_ptr(), packed.data_ptr(),
+                                                 scale.data_ptr(), mn.data_ptr(), st))
         # the widths are kept as they were at quantize time: the caller may refresh its own copy
         return BatchedPacked(self, packed, scale, mn, table, bits.clone(), plan, [t.shape for t in tensors],
                              list(self.dtypes), seeds)
@@ -139,13 +145,13 @@ class BatchedQuantizer:
             # a fresh table with x pointing at the outputs; planning it again from the same widths gives
             # the same offsets without reading anything back
             table = self._table(outs, q.seeds)
-            plan = torch.empty((2,), dtype=torch.int64, device=self.device)
+            plan = torch.empty((6,), dtype=torch.int64, device=self.device)
             st = torch.cuda.current_stream(self.device).cuda_stream
             _abi.check(lib.gact_batch_plan(table.data_ptr(), q.bits.data_ptr(), self.L, q.packed.numel(),
                                            plan.data_ptr(), st))
             _abi.check(lib.gact_dequantize_batched(table.data_ptr(), q.bits.data_ptr(), self.L, self.total_blocks,
-                                                   plan.data_ptr(), q.packed.data_ptr(), q.scale.data_ptr(),
-                                                   q.min.data_ptr(), st))
+                                                   plan.data_ptr(), self.block_map.data_ptr(), q.packed.data_ptr(),
+                                                   q.scale.data_ptr(), q.min.data_ptr(), st))
             # keep the table alive until the stream has consumed it
             q._dq_table = (table, plan)
         return outs

@@ -50,8 +50,8 @@ SIGNATURES = {
     "gact_calc_precision": (_i32, [_vp, _vp, _vp, _i64, _f64]),
     "gact_calc_precision_device": (_i32, [_vp, _vp, _vp, _i64, _f64, _vp, _vp]),
     "gact_batch_plan": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp]),
-    "gact_quantize_batched": (_i32, [_vp, _vp, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp]),
-    "gact_dequantize_batched": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "gact_quantize_batched": (_i32, [_vp, _vp, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "gact_dequantize_batched": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
 }
 
 

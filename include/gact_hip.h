@@ -105,24 +105,27 @@ typedef struct gact_batch_entry {
 } gact_batch_entry;
 
 /* Fill packed_offset (256-byte aligned, in table order) from device-resident bits.  `plan` is a device
- * array of two int64: plan[0] receives the arena bytes the table needs, plan[1] receives 1 when every
- * bits[i] is in {1,2,4,8} and plan[0] <= capacity, else 0 (the batched kernels then do nothing).
- * No counterpart in the reference. */
+ * array of six int64: plan[0] receives the arena bytes the table needs, plan[1] receives 1 when every
+ * bits[i] is in {1,2,4,8} and plan[0] <= capacity, else 0 (the batched kernels then do nothing),
+ * plan[2..5] the number of tensors at width 1, 2, 4, 8.  No counterpart in the reference. */
 int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t capacity, int64_t* plan,
                     void* stream);
 
 /* Quantize / dequantize all L tensors of the table over a grid of `total_blocks` blocks (the sum of
  * ceil(N_i/128)), each tensor at its own bits[i] read from device memory; the grid is launched once per
  * width (four launches, blocks of tensors at another width leave at once).  Scale and min of tensor i
- * are written at byte offset 4*stats_offset of their arenas.  Results equal a loop of gact_quantize /
- * gact_dequantize over the tensors (gact/gact/quantizer.py:95-142 drives the reference one tensor at a
- * time).  `plan` is the array gact_batch_plan filled. */
+ * are written at byte offset 4*stats_offset of their arenas (keep stats_offset a multiple of 8 so that
+ * the rows stay 32-byte aligned).  `block_map` (device int32[total_blocks], may be null) names the
+ * tensor of every block; without it each block searches the table.  Results equal a loop of
+ * gact_quantize / gact_dequantize over the tensors (gact/gact/quantizer.py:95-142 drives the reference
+ * one tensor at a time).  `plan` is the array gact_batch_plan filled. */
 int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
-                          int noise_mode, const int64_t* plan, void* packed_arena, void* scale_arena,
-                          void* min_arena, void* stream);
+                          int noise_mode, const int64_t* plan, const int32_t* block_map, void* packed_arena,
+                          void* scale_arena, void* min_arena, void* stream);
 int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L,
-                            int64_t total_blocks, const int64_t* plan, const void* packed_arena,
-                            const void* scale_arena, const void* min_arena, void* stream);
+                            int64_t total_blocks, const int64_t* plan, const int32_t* block_map,
+                            const void* packed_arena, const void* scale_arena, const void* min_arena,
+                            void* stream);
 
 #ifdef __cplusplus
 }
