@@ -2,15 +2,17 @@
 // rounding, bit packing, and the inverse, as hand-written HIP kernels behind a C ABI.
 //
 // Quantize: a DPP row of 16 lanes owns one "super-group", the 8/bits consecutive groups of 256
-// elements whose codes share output bytes.  Inside a group lane i of the row owns two runs of 8
-// consecutive columns, 128k + 8i .. +7 (k = 0,1).  Per-group reductions are four row_ror DPP steps that
-// never leave the row, and - because the reference packs the SAME column of 8/bits consecutive groups
-// into one byte - the lane that owns a column owns every code of that byte: packing needs no
-// cross-lane traffic at all.  8 consecutive elements are also what one Philox block feeds.
+// elements whose codes share output bytes.  Inside a group lane i of the row owns 16 columns in chunks
+// of one 16-byte load each - float: 4 chunks of 4 columns at 4i + 64m, half: 2 chunks of 8 columns at
+// 8i + 128m - so every load instruction of a row reads 256 contiguous bytes.  Per-group reductions are
+// four row_ror DPP steps that never leave the row, and - because the reference packs the SAME column of
+// 8/bits consecutive groups into one byte - the lane that owns a column owns every code of that byte:
+// packing needs no cross-lane traffic at all.  One Philox block feeds 8 consecutive elements: a half
+// chunk, or the two float chunks of a pair of neighbouring lanes (which swap the halves they need).
 //
-// Dequantize has no reduction, so a whole wave owns a super-group: lane l owns columns 4l .. 4l+3, reads
-// one dword of codes, and every store instruction of the wave writes one group contiguously; scale and
-// min are wave-uniform and come through the scalar cache.
+// Dequantize has no reduction, so a unit of 8 consecutive groups goes to a whole wave (float: lane l owns
+// columns 4l .. 4l+3) or half a wave (half: 8l .. 8l+7): one 16-byte store per lane and group, every store
+// instruction writing whole groups contiguously.
 //
 // Floating-point contract: this file is compiled with -ffp-contract=off, so every operation below is
 // the IEEE operation it spells; the fused multiply-adds of the path are written __builtin_fmaf.
@@ -33,7 +35,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define GROUP 256
-#define ROW_GROUPS 8 /* groups owned by one 16-lane row in the minimax and batched kernels */
+#define ROW_GROUPS 8 /* groups of a dequantize unit and of a minimax row */
 
 // ------------------------------------------------------------------------------------------------
 // DPP row reductions (16 lanes).  Rotating by 8, 4, 2, 1 leaves the row-wide result in every lane.

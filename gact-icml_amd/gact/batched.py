@@ -9,8 +9,6 @@ results are identical to calling ``op_quantize`` / ``op_dequantize`` tensor by t
 Grid layout: a block owns 128 groups of 256 elements whatever the width, so the grid
 (sum over tensors of ceil(N_i/128) blocks) is known on the host without knowing the widths.
 """
-import ctypes
-
 import torch
 
 from .cpp_extension import _abi
