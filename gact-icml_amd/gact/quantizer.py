@@ -79,35 +79,47 @@ class Quantizer:
 
     def quantize(self, input):
         """Pack hook.  Returns (False, tensor) | (True, True, q_mask) | (True, False, key, shape, tid)."""
-        quantize, is_dropout_mask = self.check_quantize(input)
-        if not quantize:
+        wanted, is_mask = self.check_quantize(input)
+        if not wanted:
             return False, input
-        if is_dropout_mask:
-            return True, is_dropout_mask, op_quantize_mask(input)
+        if is_mask:
+            return True, True, op_quantize_mask(input)
 
-        tid = self.tid
-        self.tid += 1
-        input_shape = input.shape
-
+        tid, self.tid = self.tid, self.tid + 1
         key = self.generate_tensor_key(input, tid)
         self.layer_key_map[tid] = key
-        if key in self.ptr_qtensor_map:
-            self.ptr_qtensor_map[key][1] += 1     # saved again: one more reference, no new codes
+        entry = self.ptr_qtensor_map.get(key)
+        if entry is not None:
+            entry[1] += 1                       # saved again: one more reference, no new codes
         else:
-            if self.iter == 0:
-                bit = self.default_bit
-                self.bits[tid] = bit
-                self.dims[tid] = input.numel()
-                self.seeds[tid] = tid
-            else:
-                bit = self.bits[tid]
-            q_inputs = op_quantize(input, bit, self.seeds[tid] + self.seed_iter)
-            if self.swap:
-                host = torch.empty(q_inputs[0].shape, dtype=q_inputs[0].dtype, device="cpu", pin_memory=True)
-                host.copy_(q_inputs[0], non_blocking=True)
-                q_inputs[0] = host
-            self.ptr_qtensor_map[key] = [q_inputs, 1, tid]
-        return True, is_dropout_mask, key, input_shape, tid
+            self.ptr_qtensor_map[key] = [self._compress(input, tid), 1, tid]
+        return True, False, key, input.shape, tid
+
+    def _compress(self, input, tid):
+        """Quantize one tensor at its current width; the first iteration fills the tables auto precision reads."""
+        if self.iter == 0:
+            self.bits[tid] = self.default_bit
+            self.dims[tid] = input.numel()
+            self.seeds[tid] = tid
+        q_inputs = op_quantize(input, self.bits[tid], self.seeds[tid] + self.seed_iter)
+        if self.swap:
+            host = torch.empty(q_inputs[0].shape, dtype=q_inputs[0].dtype, device="cpu", pin_memory=True)
+            host.copy_(q_inputs[0], non_blocking=True)
+            q_inputs[0] = host
+        return q_inputs
+
+    def _prefetch_previous(self, tid):
+        """Start copying layer tid-1's codes back to the GPU while layer tid is dequantized."""
+        self.start_prefetch_event.record()
+        with torch.cuda.stream(self.swap_in_stream):
+            if tid > 0:
+                self.start_prefetch_event.wait(self.swap_in_stream)
+                prev = self.ptr_qtensor_map.get(self.layer_key_map[tid - 1])
+                if prev is not None and not prev[0][0].is_cuda:
+                    prev[0][0] = prev[0][0].cuda(non_blocking=True)
+                    # allocated on the copy stream, consumed on the compute stream
+                    prev[0][0].record_stream(self.compute_stream)
+                self.end_prefetch_event.record()
 
     def dequantize(self, input):
         """Unpack hook: the inverse of quantize()."""
@@ -117,36 +129,25 @@ class Quantizer:
             return op_dequantize_mask(input[2])
 
         _, _, key, input_shape, tid = input
-        q_inputs, ref_cnt, key_tid = self.ptr_qtensor_map[key]
+        entry = self.ptr_qtensor_map[key]
+        q_inputs = entry[0]
 
-        if self.start_bwd and self.swap:
-            self.compute_stream.wait_stream(self.swap_out_stream)
-            self.start_bwd = False
-        if self.prefetch and self.swap:
-            self.end_prefetch_event.wait(self.compute_stream)
-        if self.swap and not q_inputs[0].is_cuda:   # swapped out and not prefetched: fetch it now
-            q_inputs[0] = q_inputs[0].cuda(non_blocking=False)
-
-        if self.prefetch and self.swap:
-            # bring the previous layer's codes back while this one is being dequantized
-            self.start_prefetch_event.record()
-            with torch.cuda.stream(self.swap_in_stream):
-                if tid > 0:
-                    self.start_prefetch_event.wait(self.swap_in_stream)
-                    previous_key = self.layer_key_map[tid - 1]
-                    if previous_key in self.ptr_qtensor_map:
-                        prev = self.ptr_qtensor_map[previous_key][0]
-                        if not prev[0].is_cuda:
-                            prev[0] = prev[0].cuda(non_blocking=True)
-                    self.end_prefetch_event.record()
+        if self.swap:
+            if self.start_bwd:
+                self.compute_stream.wait_stream(self.swap_out_stream)
+                self.start_bwd = False
+            if self.prefetch:
+                self.end_prefetch_event.wait(self.compute_stream)
+            if not q_inputs[0].is_cuda:         # swapped out and not prefetched: fetch it now
+                q_inputs[0] = q_inputs[0].cuda(non_blocking=False)
+            if self.prefetch:
+                self._prefetch_previous(tid)
 
         ret = op_dequantize(q_inputs, input_shape)
 
-        ref_cnt -= 1
-        if ref_cnt < 0:
+        entry[1] -= 1
+        if entry[1] < 0:
             raise RuntimeError("[Error] Ref count < 0 for key %r" % (key,))
-        if ref_cnt == 0:
+        if entry[1] == 0:
             del self.ptr_qtensor_map[key]
-        else:
-            self.ptr_qtensor_map[key] = [q_inputs, ref_cnt, key_tid]
         return ret
