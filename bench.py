@@ -3,7 +3,7 @@
 
 One step = one fused quantize (min/max + scale + stochastic rounding + pack) followed by one
 dequantize (unpack + affine) of one synthetic activation tensor, through the C ABI, with the input
-already resident in HBM.  The default workload is BASELINE.json's configs[1]: a ResNet-50 conv
+already resident in HBM.  The default workload is the headline one ("config2"): a ResNet-50 conv
 activation, fp32 NCHW [128,256,56,56], post-ReLU, group 256, 4 bit, stochastic rounding with Philox
 seed 42.  Bytes are the algorithmic input + output bytes of both directions:
 numel*sizeof(T) + packed bytes + 2*N*sizeof(T) per direction.
@@ -122,7 +122,7 @@ def run_workload(torch, name, steps, warmup, seed=42):
 
 
 def run_config5(torch, steps, warmup, seed=42):
-    """BASELINE config 5, the full adaptive step: 120 fp16 tensors with Swin-Tiny-like shapes, per-tensor
+    """Workload "config5", the full adaptive step: 120 fp16 tensors with Swin-Tiny-like shapes, per-tensor
     sensitivities ~LogNormal(0,2), budget 2 bits per element.  One step = greedy calc_precision on the GPU
     (widths stay in device memory), offset planning, one batched mixed-width quantize and one batched
     dequantize, all through the C ABI."""

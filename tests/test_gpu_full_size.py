@@ -1,4 +1,4 @@
-"""The five BASELINE workloads at their full sizes.
+"""The five benchmark workloads (config 1-5 of bench.py) at their full sizes.
 
 Each is checked three ways: against the CPU oracle on the same seeded input (bit-exact packed bytes,
 scale, min and dequantized values - the C oracle finishes these sizes in seconds), through size-independent

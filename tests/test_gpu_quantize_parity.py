@@ -145,7 +145,7 @@ def test_edge_groups(dtype, bits):
 
 
 def test_config1_full_size_deterministic():
-    # BASELINE config 1: fp32 [4096,1024] ~ N(0,1), seed 0, 2 bit, deterministic rounding
+    # benchmark workload config 1: fp32 [4096,1024] ~ N(0,1), seed 0, 2 bit, deterministic rounding
     torch.manual_seed(0)
     x = torch.randn(4096, 1024)
     q, ref = check_quantize(x, 2, "deterministic", seed=0)

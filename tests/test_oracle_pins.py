@@ -275,7 +275,7 @@ def test_sizes_of_the_reference_shapes():
     # [100,77] -> 7700 elements -> 31 groups; one-hot 1000x1000 -> 3907 groups (tests/test_act_quantized_ops.py)
     assert oracle.pad_groups(np.zeros((100, 77), np.float32)).shape == (31, 256)
     assert oracle.pad_groups(np.zeros((1000, 1000), np.float32)).shape == (3907, 256)
-    # BASELINE configs 1, 2 and 4 (packed bytes)
+    # benchmark workloads config 1, 2 and 4 (packed bytes)
     assert oracle.packed_len(2, 16384) == 1048576
     assert oracle.packed_len(4, 401408) == 51380224
     assert oracle.packed_len(1, 169343) == 5419008
