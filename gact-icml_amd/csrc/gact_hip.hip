@@ -40,26 +40,22 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // ------------------------------------------------------------------------------------------------
 // DPP row reductions (16 lanes).  Rotating by 8, 4, 2, 1 leaves the row-wide result in every lane.
 // ------------------------------------------------------------------------------------------------
-template <int CTRL>
-__device__ __forceinline__ float dpp_f32(float v) {
-  int x = __builtin_bit_cast(int, v);
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(x, x, CTRL, 0xf, 0xf, false));
+// Row-wide min of lo and max of hi, left in every lane of the row, with the rotated operand folded into the
+// min / max instruction itself (VOP2 DPP).  lo and hi must not be NaN (they are per-lane results that
+// started from a finite or infinite initial value).  A DPP operand has to be written two wait states before
+// it is read, five after a vector write of EXEC; the compiler's hazard pass does not look inside an asm
+// block, so the block keeps those distances itself, at both ends as well.
+#define GACT_DPP_STEP(MIN, MAX, N)                                         \
+  MIN " %0, %0, %0 row_ror:" #N " row_mask:0xf bank_mask:0xf\n\t"          \
+  MAX " %1, %1, %1 row_ror:" #N " row_mask:0xf bank_mask:0xf\n\t"
+#define GACT_DPP_ALL(MIN, MAX)                                             \
+  "s_nop 4\n\t" GACT_DPP_STEP(MIN, MAX, 8) "s_nop 0\n\t" GACT_DPP_STEP(MIN, MAX, 4) "s_nop 0\n\t" \
+  GACT_DPP_STEP(MIN, MAX, 2) "s_nop 0\n\t" GACT_DPP_STEP(MIN, MAX, 1) "s_nop 1"
+__device__ __forceinline__ void row_all_minmax(float& lo, float& hi) {
+  asm(GACT_DPP_ALL("v_min_f32_dpp", "v_max_f32_dpp") : "+v"(lo), "+v"(hi));
 }
-#define DPP_ROW_ROR(n) (0x120 + (n))
-
-__device__ __forceinline__ float row_all_min(float v) {
-  v = __builtin_fminf(v, dpp_f32<DPP_ROW_ROR(8)>(v));
-  v = __builtin_fminf(v, dpp_f32<DPP_ROW_ROR(4)>(v));
-  v = __builtin_fminf(v, dpp_f32<DPP_ROW_ROR(2)>(v));
-  v = __builtin_fminf(v, dpp_f32<DPP_ROW_ROR(1)>(v));
-  return v;
-}
-__device__ __forceinline__ float row_all_max(float v) {
-  v = __builtin_fmaxf(v, dpp_f32<DPP_ROW_ROR(8)>(v));
-  v = __builtin_fmaxf(v, dpp_f32<DPP_ROW_ROR(4)>(v));
-  v = __builtin_fmaxf(v, dpp_f32<DPP_ROW_ROR(2)>(v));
-  v = __builtin_fmaxf(v, dpp_f32<DPP_ROW_ROR(1)>(v));
-  return v;
+__device__ __forceinline__ void row_all_minmax(f16& lo, f16& hi) {
+  asm(GACT_DPP_ALL("v_min_f16_dpp", "v_max_f16_dpp") : "+v"(lo), "+v"(hi));
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -177,8 +173,9 @@ template <> struct Elem<float> {
   __device__ static __forceinline__ void group_minmax(const Store& st, float& lo_out, float& hi_out) {
     float lo = init_lo(), hi = init_hi();
     minmax(st, lo, hi);
-    lo_out = row_all_min(lo);
-    hi_out = row_all_max(hi);
+    row_all_minmax(lo, hi);
+    lo_out = lo;
+    hi_out = hi;
   }
   __device__ static __forceinline__ void store_codes(uint8_t* p, const uint32_t (&b)[4]) {
     // the reference accumulates in a uint8_t: keep the low 8 bits of every byte
@@ -260,37 +257,40 @@ template <> struct Elem<f16> {
     lo = __builtin_fminf((float)l.x, (float)l.y);
     hi = __builtin_fmaxf((float)h.x, (float)h.y);
   }
-  // min and max of the whole group, in every lane of the row: packed per-lane min / max, then ONE row
-  // reduction over the pair {min, -max} with packed min
+  // Packed min / max without the canonicalising copy the compiler puts in front of every minnum / maxnum
+  // operand: a quiet NaN operand loses against the other one, which is the reference's "NaN is ignored".
+  // (A signalling NaN, which arithmetic never produces, would be returned quieted instead.)
+  __device__ static __forceinline__ f16x2 pk_min(f16x2 a, f16x2 b) {
+    f16x2 d;
+    asm("v_pk_min_f16 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+  }
+  __device__ static __forceinline__ f16x2 pk_max(f16x2 a, f16x2 b) {
+    f16x2 d;
+    asm("v_pk_max_f16 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+  }
+  // min and max of the whole group, in every lane of the row: packed per-lane min / max from +-inf (the
+  // start values only survive in a lane whose 16 elements are all NaN), the two halves against each other,
+  // then the row reduction
   __device__ static __forceinline__ void group_minmax(const Store& st, f16& lo_out, f16& hi_out) {
-    f16x2 l = st.v[0][0], h = st.v[0][0];
+    const f16 inf = (f16)__builtin_inff();
+    f16x2 l = {inf, inf}, h = {(f16)-inf, (f16)-inf};
 #pragma unroll
     for (int k = 0; k < 2; k++)
 #pragma unroll
       for (int j = 0; j < 4; j++) {
-        if (k + j == 0) continue;
-        l = __builtin_elementwise_min(l, st.v[k][j]);
-        h = __builtin_elementwise_max(h, st.v[k][j]);
+        l = pk_min(l, st.v[k][j]);
+        h = pk_max(h, st.v[k][j]);
       }
-    // NaN elements never win a min / max; start values +-inf only matter for an all-NaN group
-    const f16 inf = (f16)__builtin_inff();
-    const f16 lmin = __builtin_elementwise_min(__builtin_elementwise_min((f16)l.x, (f16)l.y), inf);
-    const f16 hmax = __builtin_elementwise_max(__builtin_elementwise_max((f16)h.x, (f16)h.y), (f16)-inf);
-    f16x2 m = {lmin, (f16)-hmax};
-#pragma unroll
-    for (int step = 8; step >= 1; step >>= 1) {
-      const int bits = __builtin_bit_cast(int, m);
-      int other;
-      switch (step) {
-        case 8: other = __builtin_amdgcn_update_dpp(bits, bits, DPP_ROW_ROR(8), 0xf, 0xf, false); break;
-        case 4: other = __builtin_amdgcn_update_dpp(bits, bits, DPP_ROW_ROR(4), 0xf, 0xf, false); break;
-        case 2: other = __builtin_amdgcn_update_dpp(bits, bits, DPP_ROW_ROR(2), 0xf, 0xf, false); break;
-        default: other = __builtin_amdgcn_update_dpp(bits, bits, DPP_ROW_ROR(1), 0xf, 0xf, false); break;
-      }
-      m = __builtin_elementwise_min(m, __builtin_bit_cast(f16x2, other));
-    }
-    lo_out = m.x;
-    hi_out = -m.y;
+    f16 lo, hi;
+    asm("v_min_f16_sdwa %0, %1, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1"
+        : "=v"(lo) : "v"(l));
+    asm("v_max_f16_sdwa %0, %1, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1"
+        : "=v"(hi) : "v"(h));
+    row_all_minmax(lo, hi);
+    lo_out = lo;
+    hi_out = hi;
   }
   // range is a half operation; the quotient is a double narrowed to float and then to half
   __device__ static __forceinline__ f16 make_scale(f16 lo, f16 hi, int qmax) {

@@ -89,7 +89,16 @@ def dtype_code(dtype):
 
 def stream_of(t):
     """Raw HIP stream torch currently launches on for t's device."""
-    return torch.cuda.current_stream(t.device).cuda_stream
+    return torch._C._cuda_getCurrentRawStream(t.device.index)
+
+
+def call_on(device, fn, *args):
+    """Call a library entry point with `device` current (the kernels launch on the current HIP device) and
+    turn its status into RuntimeError.  With a single visible GPU there is nothing to switch."""
+    if torch.cuda.device_count() == 1:
+        return check(fn(*args))
+    with torch.cuda.device(device):
+        return check(fn(*args))
 
 
 def ptr(t):

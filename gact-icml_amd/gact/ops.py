@@ -7,7 +7,7 @@ instead of a concatenated copy.  ``op_dequantize`` writes straight into a tensor
 shape.  The extension-style entry points (minimax, pack_single_precision, unpack_single_precision)
 stay available in gact.cpp_extension for callers that use them directly.
 """
-import numpy as np
+import math
 import torch
 
 from .conf import config
@@ -58,10 +58,9 @@ def no_scheme_quantize_pack(input, q_bit, seed, *, noise=None, rng_stream=None):
                           dtype=torch.int8, device=x.device)
     q_scale = torch.empty((N, 1, 1), dtype=x.dtype, device=x.device)
     q_min = torch.empty((N, 1, 1), dtype=x.dtype, device=x.device)
-    with torch.cuda.device(x.device):
-        _abi.check(_abi.lib().gact_quantize(x.data_ptr(), _abi.dtype_code(x.dtype), x.numel(), q_bit, mode, seed,
-                                            _abi.ptr(noise), q_input.data_ptr(), q_scale.data_ptr(),
-                                            q_min.data_ptr(), None, _abi.stream_of(x)))
+    _abi.call_on(x.device, _abi.lib().gact_quantize, x.data_ptr(), _abi.dtype_code(x.dtype), x.numel(), q_bit, mode,
+                 seed, _abi.ptr(noise), q_input.data_ptr(), q_scale.data_ptr(), q_min.data_ptr(), None,
+                 _abi.stream_of(x))
     return q_input, q_scale, q_min
 
 
@@ -75,7 +74,7 @@ def dequantize_and_unpack(data, shape, q_bit, scale, mn):
         return data
 
     group_size = config.group_size
-    num_groups = (int(np.prod(shape)) + group_size - 1) // group_size
+    num_groups = (math.prod(shape) + group_size - 1) // group_size
     return ext_quantization.unpack_single_precision(data, q_bit, scale, mn, num_groups, 1, group_size)
 
 
@@ -87,7 +86,7 @@ def op_quantize_mask(input):
 def op_dequantize_mask(input):
     """gact/gact/ops.py:52-55."""
     q_mask, input_shape = input
-    output = ext_quantization.act_dequantize_dropout_mask(q_mask, np.prod(input_shape)).reshape(input_shape)
+    output = ext_quantization.act_dequantize_dropout_mask(q_mask, math.prod(input_shape)).reshape(input_shape)
     return output
 
 
@@ -103,7 +102,7 @@ def op_dequantize(input, input_shape):
     if not isinstance(q_bit, int):
         print("bits must be intergers, now bits ", q_bit)
         assert(False)
-    num_features = int(np.prod(input_shape))
+    num_features = math.prod(input_shape)
     if q_bit == 32:
         return q_input.ravel()[:num_features].reshape(*input_shape).contiguous()
 
@@ -120,8 +119,7 @@ def op_dequantize(input, input_shape):
     if q_scale.dtype != q_min.dtype:
         raise RuntimeError("expected scalar type of min to match scale")
     out = torch.empty(tuple(input_shape), dtype=q_scale.dtype, device=q_input.device)
-    with torch.cuda.device(q_input.device):
-        _abi.check(_abi.lib().gact_dequantize(q_input.data_ptr(), q_bit, q_scale.data_ptr(), q_min.data_ptr(),
-                                              _abi.dtype_code(q_scale.dtype), num_features, out.data_ptr(),
-                                              _abi.stream_of(q_input)))
+    _abi.call_on(q_input.device, _abi.lib().gact_dequantize, q_input.data_ptr(), q_bit, q_scale.data_ptr(),
+                 q_min.data_ptr(), _abi.dtype_code(q_scale.dtype), num_features, out.data_ptr(),
+                 _abi.stream_of(q_input))
     return out
