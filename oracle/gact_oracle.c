@@ -19,9 +19,13 @@
  *                           reference's one-hot round trips
  *   philox4x32_10  pinned   Random123 known-answer vectors
  *   reference noise stream (cuRAND Philox state walk + uniform map):
- *                  PARITY UNPINNED - the reference holds no vector for it and
- *                  cuRAND is not in this image; restated from its published
- *                  header semantics
+ *                  the reference holds no vector for it and cuRAND is not in
+ *                  this image; restated from its published header semantics
+ *                  and pinned on the GPU against hipRAND's cuRAND-compatible
+ *                  Philox as torch's device generator draws it (seed, subsequence,
+ *                  offset -> key / counter, word order, next block, uniform map:
+ *                  tests/test_gpu_philox_library.py).  PARITY UNPINNED only in
+ *                  that cuRAND itself was never run
  *   fast noise stream        our own definition, no reference counterpart
  *   calc_precision pinned   against the reference's calc_precision.cc compiled
  *                           as-is into oracle/_ref (when built) + hand cases
