@@ -148,3 +148,61 @@ def test_auto_precision_training_is_identical_with_and_without_swap():
     assert bits == bits_s
     assert set(bits.values()) <= {1, 2, 4, 8, 32} and len(bits) >= 4
     assert all(l == l for l in base)              # no NaN
+
+
+class MaskedScale(torch.autograd.Function):
+    """Dropout as the torch versions the reference targets saved it: a uint8 0/1 mask kept for backward."""
+
+    @staticmethod
+    def forward(ctx, x, mask):
+        ctx.save_for_backward(mask)
+        return x * mask
+
+    @staticmethod
+    def backward(ctx, g):
+        (mask,) = ctx.saved_tensors
+        return g * mask, None
+
+
+def test_saved_uint8_mask_takes_the_one_bit_mask_kernels(monkeypatch):
+    """quantizer.py:52-55,102-104 of the reference: a saved uint8 tensor holding only 0 and 1 is packed to one
+    bit per element; the backward pass must get the very same mask back."""
+    import gact.quantizer as quantizer_mod
+
+    calls = {"pack": 0, "unpack": 0, "words": 0}
+    real_qm, real_dm = quantizer_mod.op_quantize_mask, quantizer_mod.op_dequantize_mask
+
+    def qm(t):
+        q = real_qm(t)
+        calls["pack"] += 1
+        calls["words"] = q[0].numel()
+        assert q[0].dtype == torch.int32
+        return q
+
+    def dm(q):
+        calls["unpack"] += 1
+        return real_dm(q)
+
+    monkeypatch.setattr(quantizer_mod, "op_quantize_mask", qm)
+    monkeypatch.setattr(quantizer_mod, "op_dequantize_mask", dm)
+    torch.manual_seed(11)
+    lin = nn.Linear(300, 77).cuda()
+    x = torch.randn(100, 300, device="cuda")
+    mask = (torch.rand(100, 77, device="cuda") < 0.7).to(torch.uint8)       # 7700 elements: a ragged last word
+    out = MaskedScale.apply(lin(x), mask)
+    out.sum().backward()
+    exact = lin.weight.grad.clone()
+    lin.zero_grad()
+
+    gact.set_optimization_level("L1.1")
+    ctl = Controller(lin)
+    ctl.install_hook()
+    try:
+        out = MaskedScale.apply(lin(x), mask)
+        out.sum().backward()
+    finally:
+        ctl.uninstall_hook()
+    assert calls == {"pack": 1, "unpack": 1, "words": (7700 + 31) // 32}
+    # the mask comes back exactly; the only lossy tensor is the 8-bit input of the linear layer
+    assert torch.equal(lin.bias.grad, mask.float().sum(0))
+    assert ((lin.weight.grad - exact).norm() / exact.norm()).item() < 0.02
