@@ -1215,8 +1215,14 @@ inline void row_grid(int64_t rows, dim3* grid, dim3* block, int threads = 256) {
 // Workgroup size of the quantize kernel.  A row's work grows with 8/bits groups; the long-running
 // low-width rows schedule better as single-wave workgroups (measured: float 2 bit 5.7 -> 6.2 TB/s,
 // 1 bit 5.4 -> 6.0 TB/s), the short high-width ones as four waves.
+#ifndef GACT_Q_WIDE_F32
+#define GACT_Q_WIDE_F32 8
+#endif
+#ifndef GACT_Q_WIDE_F16
+#define GACT_Q_WIDE_F16 4
+#endif
 inline int quantize_threads(int bits, size_t elem_size) {
-  const int wide_from = elem_size == 4 ? 8 : 4;
+  const int wide_from = elem_size == 4 ? GACT_Q_WIDE_F32 : GACT_Q_WIDE_F16;
   return bits >= wide_from ? 256 : 64;
 }
 inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8 / bits); }

@@ -246,3 +246,45 @@ def test_more_than_2_to_31_elements(bits):
         rrow, rni = divmod(n_local, wpt)
         want = (ref[0][rrow * 256: rrow * 256 + 256] >> (rni * bits)) & (2 ** bits - 1)
         assert np.array_equal(got, want)
+
+
+def random_case(rng):
+    dtype = DTYPES[rng.integers(2)]
+    bits = BITS[rng.integers(4)]
+    mode = list(MODES)[rng.integers(3)]
+    numel = int(rng.choice([rng.integers(1, 600), rng.integers(600, 40000), 256 * rng.integers(1, 70)]))
+    magnitude = 10.0 ** rng.uniform(-6, 4 if dtype == torch.float32 else 3)
+    offset = rng.choice([0.0, 1.0, -3.0, 100.0]) * magnitude
+    x = rng.standard_normal(numel) * magnitude + offset
+    kind = rng.integers(6)
+    if kind == 0:
+        x = np.maximum(x - offset, 0.0)                    # post-ReLU: many exact zeros, -0.0 never
+    elif kind == 1:
+        x = np.round(x / magnitude) * magnitude            # few distinct values, many ties
+    elif kind == 2:
+        x[rng.random(numel) < 0.05] = np.nan               # scattered NaN
+    elif kind == 3 and numel >= 512:
+        g = rng.integers(numel // 256)
+        x[g * 256:(g + 1) * 256] = np.nan                  # a whole group of NaN
+        x[(g ^ 1) * 256 + 8 * 3:(g ^ 1) * 256 + 8 * 3 + 8] = np.nan   # and all of one lane's first chunk
+    elif kind == 4:
+        x = -np.abs(x)                                     # negative only, -0.0 possible after the cast
+    return torch.from_numpy(x).to(dtype), bits, mode
+
+
+def test_random_cases_against_the_oracle():
+    rng = np.random.default_rng(2024)
+    for case in range(150):
+        x, bits, mode = random_case(rng)
+        seed = int(rng.integers(0, 2 ** 31 - 1))
+        try:
+            q, ref = check_quantize(x, bits, mode, seed)
+            out = ops.op_dequantize(q, x.shape).cpu().numpy()
+            want = oracle.op_dequantize(ref, tuple(x.shape))
+            np.testing.assert_array_equal(np.isnan(out), np.isnan(want))
+            m = ~np.isnan(want)
+            it = np.uint16 if out.dtype == np.float16 else np.uint32
+            np.testing.assert_array_equal(out[m].view(it), want[m].view(it))
+        except AssertionError as e:
+            raise AssertionError("case %d: dtype %s bits %d stream %s numel %d seed %d: %s"
+                                 % (case, x.dtype, bits, mode, x.numel(), seed, e))
