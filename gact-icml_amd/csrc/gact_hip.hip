@@ -213,6 +213,12 @@ template <> struct Elem<float> {
     float q = d.fast ? div_by_reciprocal((float)c, d.s, d.r) : (float)c / d.s;
     return q + d.mn;
   }
+  // quotient -> output; one table entry T(c)/scale + min; 32 bits fetched from another lane -> value
+  __device__ static __forceinline__ float finish(float q, float mn) { return q + mn; }
+  __device__ static __forceinline__ uint32_t table_entry(float c, float s, float mn) {
+    return __builtin_bit_cast(uint32_t, c / s + mn);
+  }
+  __device__ static __forceinline__ float from_bits(uint32_t b) { return __builtin_bit_cast(float, b); }
   static constexpr int kDqWidth = 4;  // columns per dequantize lane: one 16-byte store
   __device__ static __forceinline__ void store_dq(float* p, const float (&v)[4]) {
     f32x4 a = {v[0], v[1], v[2], v[3]};
@@ -349,6 +355,11 @@ template <> struct Elem<f16> {
     float q = d.fast ? div_by_reciprocal((float)c, d.s, d.r) : (float)c / d.s;
     return (f16)q + d.mn;
   }
+  __device__ static __forceinline__ f16 finish(float q, f16 mn) { return (f16)q + mn; }
+  __device__ static __forceinline__ uint32_t table_entry(float c, f16 s, f16 mn) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (f16)((f16)(c / (float)s) + mn));
+  }
+  __device__ static __forceinline__ f16 from_bits(uint32_t b) { return __builtin_bit_cast(f16, (uint16_t)b); }
   static constexpr int kDqWidth = 8;  // columns per dequantize lane: one 16-byte store
   __device__ static __forceinline__ void store_dq(f16* p, const f16 (&v)[8]) {
     f16x8 a;
@@ -572,16 +583,36 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
 // columns W*l .. W*l+W-1 of every group (one 16-byte store per group), so 256/W lanes cover a group:
 // a whole wave per unit for float, half a wave for half.  All code words are loaded first, then the 8
 // groups are written, each store instruction covering whole groups contiguously.
-// quantization_cuda_kernel.cu:149-177.
+// The values follow quantization_cuda_kernel.cu:149-177: T(code) / scale with a real division, + min.
+// 1, 2 and 4 bit tabulate the 2^BITS values of a group once and look them up; 8 bit computes
+// them per element from one correctly rounded reciprocal per group.
 // ------------------------------------------------------------------------------------------------
+// value of lane g (0..7) of the row in every lane of the row; g is a constant once the caller's loop is unrolled
+__device__ __forceinline__ float row_bcast_at(float v, int g) {
+  switch (g) {
+    case 0: return row_bcast<0>(v);
+    case 1: return row_bcast<1>(v);
+    case 2: return row_bcast<2>(v);
+    case 3: return row_bcast<3>(v);
+    case 4: return row_bcast<4>(v);
+    case 5: return row_bcast<5>(v);
+    case 6: return row_bcast<6>(v);
+    default: return row_bcast<7>(v);
+  }
+}
+
 template <typename T, int BITS, int SGS>
 __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
                                                 const T* __restrict__ mn, int64_t numel, int64_t N, int64_t unit,
                                                 int l, T* __restrict__ out) {
   constexpr int WPT = 8 / BITS;
   constexpr int W = Elem<T>::kDqWidth;
+  constexpr int G = SGS * WPT;
+  static_assert(G == ROW_GROUPS, "a dequantize unit is 8 groups");
   const int64_t sg0 = unit * SGS;
   const int64_t n_sg = (N + WPT - 1) / WPT;
+  const int64_t g0 = sg0 * WPT;
+  const int rl = l & 15;  // lane within its 16-lane row
   uint32_t w[SGS][W / 4];
 #pragma unroll
   for (int it = 0; it < SGS; it++) {
@@ -596,10 +627,51 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
       w[it][W / 4 - 1] = t.y;
     }
   }
-  // scale and min of the unit's groups: 16-byte loads when the whole unit exists and the arrays allow it
-  constexpr int G = SGS * WPT;
+
+  if constexpr (BITS <= 4) {
+    // A group has only 2^BITS distinct outputs T(c)/scale + min.  The 16 lanes of a row tabulate them - one
+    // entry per lane, 16/2^BITS groups per pass, with the real division and the real sum - and every element
+    // then fetches its value from the lane that holds it (ds_bpermute: the LDS crossbar, no LDS memory).
+    // 2 vector instructions per element instead of 6, and the division runs once per table entry.
+    constexpr int ENT = 1 << BITS, GPP = 16 / ENT, PASSES = G / GPP;
+    const float cf = (float)(rl & (ENT - 1));
+    uint32_t tab[PASSES];
+#pragma unroll
+    for (int p = 0; p < PASSES; p++) {
+      const int64_t g = g0 + p * GPP + rl / ENT;
+      const bool live = g < N;
+      tab[p] = Elem<T>::table_entry(cf, live ? scale[g] : (T)1, live ? mn[g] : (T)0);
+    }
+    const uint32_t rowbase = threadIdx.x & 48u;
+#pragma unroll
+    for (int it = 0; it < SGS; it++) {
+#pragma unroll
+      for (int ni = 0; ni < WPT; ni++) {
+        const int64_t n = (sg0 + it) * WPT + ni;
+        if (n < N) {
+          const int g = it * WPT + ni;
+          const uint32_t base4 = (rowbase + (uint32_t)(g % GPP) * ENT) << 2;
+          T v[W];
+#pragma unroll
+          for (int e = 0; e < W; e++) {
+            const uint32_t c = __builtin_amdgcn_ubfe(w[it][e >> 2], 8 * (e & 3) + ni * BITS, BITS);
+            v[e] = Elem<T>::from_bits((uint32_t)__builtin_amdgcn_ds_bpermute((int)((c << 2) + base4), (int)tab[g / GPP]));
+          }
+          const int64_t at = n * GROUP + W * l;
+          if (n * GROUP + GROUP <= numel) {
+            Elem<T>::store_dq(out + at, v);
+          } else {
+#pragma unroll
+            for (int e = 0; e < W; e++)
+              if (at + e < numel) out[at + e] = v[e];
+          }
+        }
+      }
+    }
+    return;
+  } else {
+  // 8 bit.  scale and min of the unit's groups: 16-byte loads when the whole unit exists and the arrays allow it
   constexpr int PER16 = 16 / (int)sizeof(T);
-  const int64_t g0 = sg0 * WPT;
   T sv[G], mv[G];
   if (G % PER16 == 0 && g0 + G <= N &&
       ((reinterpret_cast<uintptr_t>(scale + g0) | reinterpret_cast<uintptr_t>(mn + g0)) & 15u) == 0) {
@@ -621,29 +693,42 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
       mv[g] = g0 + g < N ? mn[g0 + g] : (T)0;
     }
   }
+  // one correctly rounded reciprocal per group and row instead of one per group and lane: row lane j takes
+  // group j & 7 and the row shares the results; when any scale of the wave is outside the range the
+  // reciprocal form is valid for, the wave takes the plain division instead
+  const int64_t gm = g0 + (rl & 7);
+  const float s_mine = gm < N ? (float)scale[gm] : 1.0f;
+  const float r_mine = 1.0f / s_mine;
+  const bool by_reciprocal = __builtin_amdgcn_ballot_w64(!reciprocal_safe(s_mine)) == 0;
 #pragma unroll
   for (int it = 0; it < SGS; it++) {
-#pragma unroll
-    for (int ni = 0; ni < WPT; ni++) {
-      const int64_t n = (sg0 + it) * WPT + ni;
-      if (n < N) {
-        const typename Elem<T>::Dq d = Elem<T>::dq_prepare(sv[it * WPT + ni], mv[it * WPT + ni]);
-        T v[W];
+    const int64_t n = sg0 + it;
+    if (n < N) {
+      T v[W];
+      if (by_reciprocal) {
+        const float sf = (float)sv[it], r = row_bcast_at(r_mine, it);
 #pragma unroll
         for (int e = 0; e < W; e++) {
-          int c = (int)__builtin_amdgcn_ubfe(w[it][e >> 2], 8 * (e & 3) + ni * BITS, BITS);
-          v[e] = Elem<T>::decode(c, d);
+          const int c = (int)__builtin_amdgcn_ubfe(w[it][e >> 2], 8 * (e & 3), 8);
+          v[e] = Elem<T>::finish(div_by_reciprocal((float)c, sf, r), mv[it]);
         }
-        const int64_t at = n * GROUP + W * l;
-        if (n * GROUP + GROUP <= numel) {
-          Elem<T>::store_dq(out + at, v);
-        } else {
+      } else {
 #pragma unroll
-          for (int e = 0; e < W; e++)
-            if (at + e < numel) out[at + e] = v[e];
+        for (int e = 0; e < W; e++) {
+          const int c = (int)__builtin_amdgcn_ubfe(w[it][e >> 2], 8 * (e & 3), 8);
+          v[e] = Elem<T>::finish((float)c / (float)sv[it], mv[it]);
         }
       }
+      const int64_t at = n * GROUP + W * l;
+      if (n * GROUP + GROUP <= numel) {
+        Elem<T>::store_dq(out + at, v);
+      } else {
+#pragma unroll
+        for (int e = 0; e < W; e++)
+          if (at + e < numel) out[at + e] = v[e];
+      }
     }
+  }
   }
 }
 
@@ -703,11 +788,26 @@ __device__ __forceinline__ void minimax_row(const T* __restrict__ x, int64_t N, 
 // Single-tensor kernels.
 // ------------------------------------------------------------------------------------------------
 // groups a single-tensor dequantize unit (a wave for float, half a wave for half) covers
-#ifndef GACT_DQ_GROUPS
-#define GACT_DQ_GROUPS 8
+__host__ __device__ constexpr int dq_supergroups(int bits) { return ROW_GROUPS / (8 / bits); }
+
+// Workgroups go to the 8 XCDs round-robin (workgroup b runs on XCD b % 8) and every XCD streams through its
+// own L2.  With the plain mapping an XCD sees every 8th tile, i.e. addresses in which three bits never
+// change; handing each XCD runs of RUN consecutive tiles instead lets its writes leave as contiguous
+// stretches (pure-write kernels with 8 KB per wave: 5.4 -> 6.2 TB/s).  The tail that does not fill a
+// round of 8 * RUN tiles keeps the plain mapping.  RUN = 0 switches the remapping off.
+#ifndef GACT_XCD_RUN_DQ
+#define GACT_XCD_RUN_DQ 16
 #endif
-__host__ __device__ constexpr int dq_supergroups(int bits) {
-  return GACT_DQ_GROUPS / (8 / bits) > 0 ? GACT_DQ_GROUPS / (8 / bits) : 1;
+#ifndef GACT_XCD_RUN_Q
+#define GACT_XCD_RUN_Q 32 /* quantize, 4 and 8 bit (2-3 % there; the 1 and 2 bit kernels lose with it) */
+#endif
+template <uint32_t RUN>
+__device__ __forceinline__ uint32_t xcd_tile(uint32_t b, uint32_t nb) {
+  if (RUN == 0) return b;
+  constexpr uint32_t XCDS = 8, ROUND = XCDS * (RUN ? RUN : 1);
+  if (b >= nb / ROUND * ROUND) return b;
+  const uint32_t q = b / XCDS, x = b % XCDS;
+  return ((q / (RUN ? RUN : 1)) * XCDS + x) * (RUN ? RUN : 1) + q % (RUN ? RUN : 1);
 }
 
 // One super-group per 16-lane row: short waves, many of them.
@@ -715,7 +815,8 @@ template <typename T, int BITS, int NOISE, bool GIVEN>
 __global__ void __launch_bounds__(256)
 quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
                 T* __restrict__ scale_out, T* mn_io, T* mx_io, uint64_t seed, const float* __restrict__ noise) {
-  const int64_t sg = (int64_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
+  constexpr uint32_t RUN = BITS >= 4 ? GACT_XCD_RUN_Q : 0;
+  const int64_t sg = (int64_t)xcd_tile<RUN>(blockIdx.x, gridDim.x) * (blockDim.x >> 4) + (threadIdx.x >> 4);
   if (sg * (8 / BITS) >= N) return;
   quantize_supergroup<T, BITS, NOISE, GIVEN>(x, numel, N, sg, threadIdx.x & 15, packed, scale_out, mn_io, mx_io,
                                              (uint32_t)seed, (uint32_t)(seed >> 32), noise);
@@ -726,9 +827,9 @@ __global__ void __launch_bounds__(256)
 dequantize_kernel(const uint8_t* __restrict__ packed, const T* __restrict__ scale, const T* __restrict__ mn,
                   int64_t numel, int64_t N, T* __restrict__ out) {
   constexpr int LPU = GROUP / Elem<T>::kDqWidth;  // lanes per unit of 8 groups: 64 (float) or 32 (half)
-  const int64_t unit = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / LPU;
+  const int64_t unit = ((int64_t)xcd_tile<GACT_XCD_RUN_DQ>(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x) / LPU;
   constexpr int SGS = dq_supergroups(BITS);
-  if (unit * (SGS * (8 / BITS)) >= N) return;
+  if (unit * ROW_GROUPS >= N) return;
   dequantize_unit<T, BITS, SGS>(packed, scale, mn, numel, N, unit, threadIdx.x % LPU, out);
 }
 
@@ -1272,7 +1373,7 @@ int dispatch_dequantize(int bits, const uint8_t* packed, const T* scale, const T
                         hipStream_t stream) {
   // a unit of 8 groups takes 256 / (16 / sizeof(T)) lanes
   const int64_t units_per_block = 256 / (GROUP / (16 / (int64_t)sizeof(T)));
-  const int64_t unit_groups = (int64_t)dq_supergroups(bits) * (8 / bits);
+  const int64_t unit_groups = ROW_GROUPS;
   const dim3 grid((unsigned)(((N + unit_groups - 1) / unit_groups + units_per_block - 1) / units_per_block)), block(256);
   switch (bits) {
     case 1: hipLaunchKernelGGL((dequantize_kernel<T, 1>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
