@@ -12,7 +12,11 @@
 //
 // Dequantize has no reduction, so a unit of 8 consecutive groups goes to a whole wave (float: lane l owns
 // columns 4l .. 4l+3) or half a wave (half: 8l .. 8l+7): one 16-byte store per lane and group, every store
-// instruction writing whole groups contiguously.
+// instruction writing whole groups contiguously.  At 1, 2 and 4 bit the 2^bits possible values of a group
+// are tabulated once in the lanes of a row and fetched with ds_bpermute.
+//
+// Workgroups are dealt to the 8 XCDs round-robin; xcd_tile() reorders the tiles so that each XCD's L2
+// streams runs of consecutive tiles.
 //
 // Floating-point contract: this file is compiled with -ffp-contract=off, so every operation below is
 // the IEEE operation it spells; the fused multiply-adds of the path are written __builtin_fmaf.
@@ -251,18 +255,6 @@ template <> struct Elem<f16> {
   __device__ static __forceinline__ float init_lo() { return __builtin_inff(); }  // half(1e30) is +inf
   __device__ static __forceinline__ float init_hi() { return -__builtin_inff(); }
   __device__ static __forceinline__ f16 from_float(float v) { return (f16)v; }
-  __device__ static __forceinline__ void minmax(const Store& st, float& lo, float& hi) {
-    f16x2 l = {(f16)lo, (f16)lo}, h = {(f16)hi, (f16)hi};
-#pragma unroll
-    for (int k = 0; k < 2; k++)
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        l = __builtin_elementwise_min(l, st.v[k][j]);
-        h = __builtin_elementwise_max(h, st.v[k][j]);
-      }
-    lo = __builtin_fminf((float)l.x, (float)l.y);
-    hi = __builtin_fmaxf((float)h.x, (float)h.y);
-  }
   // Packed min / max without the canonicalising copy the compiler puts in front of every minnum / maxnum
   // operand: a quiet NaN operand loses against the other one, which is the reference's "NaN is ignored".
   // (A signalling NaN, which arithmetic never produces, would be returned quieted instead.)
@@ -749,18 +741,19 @@ __device__ __forceinline__ void quantize_block128(const T* __restrict__ x, int64
                                                  (uint32_t)seed, (uint32_t)(seed >> 32), nullptr);
   }
 }
-// Dequantize: the 16 units of 8 groups of the block go round-robin over the block's unit slots
-// (4 waves for float, 8 half-waves for half).
+// Dequantize: two workgroups share a block of 128 groups, 8 units of 8 groups each, so that a unit slot
+// (a wave for float, half a wave for half) gets one unit for half and two for float - several units in a
+// row per wave cost 10-20 %.
 template <typename T, int BITS>
 __device__ __forceinline__ void dequantize_block128(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
                                                     const T* __restrict__ mn, int64_t numel, int64_t N, int64_t lb,
-                                                    T* __restrict__ out) {
+                                                    int half, T* __restrict__ out) {
   constexpr int LPU = GROUP / Elem<T>::kDqWidth;  // lanes per unit
   constexpr int SLOTS = 256 / LPU;
   const int slot = threadIdx.x / LPU, l = threadIdx.x % LPU;
 #pragma unroll 1
-  for (int it = 0; it < 16 / SLOTS; it++) {
-    const int64_t unit = lb * 16 + it * SLOTS + slot;
+  for (int it = 0; it < 8 / SLOTS; it++) {
+    const int64_t unit = lb * 16 + half * 8 + it * SLOTS + slot;
     if (unit * ROW_GROUPS < N) dequantize_unit<T, BITS, BITS>(packed, scale, mn, numel, N, unit, l, out);
   }
 }
@@ -1252,8 +1245,8 @@ __device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ t
   return lo;
 }
 
-// One launch per width: blocks whose tensor has another width leave at once, so every width gets a
-// kernel with its own register allocation.
+// Quantize, one launch per width: blocks whose tensor has another width leave at once, so every width gets a
+// kernel with its own register allocation (176 registers at 1 bit float, 39 at 8 bit).
 template <int BITS, int NOISE>
 __global__ void __launch_bounds__(256)
 quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
@@ -1276,25 +1269,38 @@ quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_
     quantize_block128<f16, BITS, NOISE>((const f16*)ent.x, ent.numel, N, lb, packed, (f16*)sc, (f16*)mn, ent.seed);
 }
 
+// Dequantize, one launch for all widths (every width fits 60 registers): the width of a block's tensor is read
+// from device memory and selects the code path, so no workgroup is launched only to leave.
 template <int BITS>
+__device__ __forceinline__ void dequantize_batched_block(const gact_batch_entry& ent, int64_t lb, int half,
+                                                         const uint8_t* packed, const uint8_t* sc, const uint8_t* mn) {
+  const int64_t N = (ent.numel + GROUP - 1) / GROUP;
+  if (ent.dtype == GACT_F32)
+    dequantize_block128<float, BITS>(packed, (const float*)sc, (const float*)mn, ent.numel, N, lb, half, (float*)ent.x);
+  else
+    dequantize_block128<f16, BITS>(packed, (const f16*)sc, (const f16*)mn, ent.numel, N, lb, half, (f16*)ent.x);
+}
+// grid: two workgroups per block of 128 groups
 __global__ void __launch_bounds__(256)
 dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
                           const int64_t* __restrict__ plan, const int32_t* __restrict__ block_map,
                           const uint8_t* __restrict__ packed_arena, const uint8_t* __restrict__ scale_arena,
                           const uint8_t* __restrict__ min_arena) {
-  if (plan[1] == 0 || plan[2 + (BITS == 1 ? 0 : BITS == 2 ? 1 : BITS == 4 ? 2 : 3)] == 0) return;
-  const int t = block_map ? block_map[blockIdx.x] : batch_find(table, L, blockIdx.x);
-  if (bits[t] != BITS) return;
+  if (plan[1] == 0) return;
+  const int64_t block = blockIdx.x >> 1;
+  const int half = blockIdx.x & 1;
+  const int t = block_map ? block_map[block] : batch_find(table, L, block);
   const gact_batch_entry ent = table[t];
-  const int64_t N = (ent.numel + GROUP - 1) / GROUP;
-  const int64_t lb = (int64_t)blockIdx.x - ent.first_block;
+  const int64_t lb = block - ent.first_block;
   const uint8_t* packed = packed_arena + ent.packed_offset;
   const uint8_t* sc = scale_arena + ent.stats_offset * 4;
   const uint8_t* mn = min_arena + ent.stats_offset * 4;
-  if (ent.dtype == GACT_F32)
-    dequantize_block128<float, BITS>(packed, (const float*)sc, (const float*)mn, ent.numel, N, lb, (float*)ent.x);
-  else
-    dequantize_block128<f16, BITS>(packed, (const f16*)sc, (const f16*)mn, ent.numel, N, lb, (f16*)ent.x);
+  switch (bits[t]) {
+    case 1: dequantize_batched_block<1>(ent, lb, half, packed, sc, mn); break;
+    case 2: dequantize_batched_block<2>(ent, lb, half, packed, sc, mn); break;
+    case 4: dequantize_batched_block<4>(ent, lb, half, packed, sc, mn); break;
+    default: dequantize_batched_block<8>(ent, lb, half, packed, sc, mn); break;
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1631,21 +1637,13 @@ int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, in
 int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
                             const int64_t* plan, const int32_t* block_map, const void* packed_arena,
                             const void* scale_arena, const void* min_arena, void* stream) {
-  if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x7fffffffLL) return GACT_EINVAL;
+  if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x3fffffffLL) return GACT_EINVAL;
   if (L == 0 || total_blocks == 0) return GACT_OK;
   if (!table || !bits || !plan || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena)) return GACT_EALIGN;
-  const dim3 grid((unsigned)total_blocks), block(256);
-  hipStream_t s = (hipStream_t)stream;
-#define GACT_LAUNCH_DB(B)                                                                                    \
-  hipLaunchKernelGGL((dequantize_batched_kernel<B>), grid, block, 0, s, table, bits, (int)L, plan,           \
-                     block_map, (const uint8_t*)packed_arena, (const uint8_t*)scale_arena,                 \
-                     (const uint8_t*)min_arena)
-  GACT_LAUNCH_DB(1);
-  GACT_LAUNCH_DB(2);
-  GACT_LAUNCH_DB(4);
-  GACT_LAUNCH_DB(8);
-#undef GACT_LAUNCH_DB
+  const dim3 grid((unsigned)(2 * total_blocks)), block(256);
+  hipLaunchKernelGGL(dequantize_batched_kernel, grid, block, 0, (hipStream_t)stream, table, bits, (int)L, plan, block_map,
+                     (const uint8_t*)packed_arena, (const uint8_t*)scale_arena, (const uint8_t*)min_arena);
   return launch_status();
 }
 

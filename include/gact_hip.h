@@ -112,8 +112,8 @@ int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int
                     void* stream);
 
 /* Quantize / dequantize all L tensors of the table over a grid of `total_blocks` blocks (the sum of
- * ceil(N_i/128)), each tensor at its own bits[i] read from device memory; the grid is launched once per
- * width (four launches, blocks of tensors at another width leave at once).  Scale and min of tensor i
+ * ceil(N_i/128)), each tensor at its own bits[i] read from device memory (quantize launches the grid once
+ * per width, blocks of tensors at another width leave at once; dequantize is one launch).  Scale and min of tensor i
  * are written at byte offset 4*stats_offset of their arenas (keep stats_offset a multiple of 8 so that
  * the rows stay 32-byte aligned).  `block_map` (device int32[total_blocks], may be null) names the
  * tensor of every block; without it each block searches the table.  Results equal a loop of
