@@ -187,8 +187,8 @@ def run_config5(torch, steps, warmup, seed=42):
     def quantize():
         _abi.check(lib.gact_batch_plan(table_q.data_ptr(), bits.data_ptr(), L, packed.numel(), plan.data_ptr(), st))
         _abi.check(lib.gact_quantize_batched(table_q.data_ptr(), bits.data_ptr(), L, bq.total_blocks, _abi.NOISE_FAST,
-                                             plan.data_ptr(), bq.block_map.data_ptr(), packed.data_ptr(), sc.data_ptr(),
-                                             mn.data_ptr(), st))
+                                             bq.dtype_mask, plan.data_ptr(), bq.block_map.data_ptr(), packed.data_ptr(),
+                                             sc.data_ptr(), mn.data_ptr(), st))
 
     def dequantize():
         _abi.check(lib.gact_batch_plan(table_d.data_ptr(), bits.data_ptr(), L, packed.numel(), plan.data_ptr(), st))

@@ -1245,9 +1245,10 @@ __device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ t
   return lo;
 }
 
-// Quantize, one launch per width: blocks whose tensor has another width leave at once, so every width gets a
-// kernel with its own register allocation (176 registers at 1 bit float, 39 at 8 bit).
-template <int BITS, int NOISE>
+// Quantize, one launch per width and element type: blocks whose tensor has another width or type leave at once,
+// so every combination gets a kernel with its own register allocation (176 registers at 1 bit float, 117 at
+// 1 bit half, 34 at 8 bit half).
+template <typename T, int BITS, int NOISE>
 __global__ void __launch_bounds__(256)
 quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
                         const int64_t* __restrict__ plan, const int32_t* __restrict__ block_map,
@@ -1258,15 +1259,12 @@ quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_
   const int t = block_map ? block_map[blockIdx.x] : batch_find(table, L, blockIdx.x);
   if (bits[t] != BITS) return;
   const gact_batch_entry ent = table[t];
+  if (ent.dtype != (sizeof(T) == 4 ? GACT_F32 : GACT_F16)) return;
   const int64_t N = (ent.numel + GROUP - 1) / GROUP;
   const int64_t lb = (int64_t)blockIdx.x - ent.first_block;
-  uint8_t* packed = packed_arena + ent.packed_offset;
-  uint8_t* sc = scale_arena + ent.stats_offset * 4;
-  uint8_t* mn = min_arena + ent.stats_offset * 4;
-  if (ent.dtype == GACT_F32)
-    quantize_block128<float, BITS, NOISE>((const float*)ent.x, ent.numel, N, lb, packed, (float*)sc, (float*)mn, ent.seed);
-  else
-    quantize_block128<f16, BITS, NOISE>((const f16*)ent.x, ent.numel, N, lb, packed, (f16*)sc, (f16*)mn, ent.seed);
+  quantize_block128<T, BITS, NOISE>((const T*)ent.x, ent.numel, N, lb, packed_arena + ent.packed_offset,
+                                    (T*)(scale_arena + ent.stats_offset * 4), (T*)(min_arena + ent.stats_offset * 4),
+                                    ent.seed);
 }
 
 // Dequantize, one launch for all widths (every width fits 60 registers): the width of a block's tensor is read
@@ -1609,21 +1607,32 @@ int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int
 }
 
 int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
-                          int noise_mode, const int64_t* plan, const int32_t* block_map, void* packed_arena,
-                          void* scale_arena, void* min_arena, void* stream) {
+                          int noise_mode, int dtypes, const int64_t* plan, const int32_t* block_map,
+                          void* packed_arena, void* scale_arena, void* min_arena, void* stream) {
   if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x7fffffffLL) return GACT_EINVAL;
   if (noise_mode != GACT_NOISE_CONST && noise_mode != GACT_NOISE_REF && noise_mode != GACT_NOISE_FAST)
     return GACT_EINVAL;  // injected noise is a single-tensor test mode
+  if (dtypes < 0 || dtypes > GACT_DTYPES_ALL) return GACT_EINVAL;
+  if (dtypes == 0) dtypes = GACT_DTYPES_ALL;
   if (L == 0 || total_blocks == 0) return GACT_OK;
   if (!table || !bits || !plan || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena)) return GACT_EALIGN;
   const dim3 grid((unsigned)total_blocks), block(256);
   hipStream_t s = (hipStream_t)stream;
-#define GACT_LAUNCH_QB(B, M)                                                                                  \
-  hipLaunchKernelGGL((quantize_batched_kernel<B, M>), grid, block, 0, s, table, bits, (int)L, plan,          \
+#define GACT_LAUNCH_QB(T, B, M)                                                                               \
+  hipLaunchKernelGGL((quantize_batched_kernel<T, B, M>), grid, block, 0, s, table, bits, (int)L, plan,       \
                      block_map, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena)
-#define GACT_LAUNCH_QB_ALL(M) \
-  do { GACT_LAUNCH_QB(1, M); GACT_LAUNCH_QB(2, M); GACT_LAUNCH_QB(4, M); GACT_LAUNCH_QB(8, M); } while (0)
+#define GACT_LAUNCH_QB_ALL(M)                                                                                 \
+  do {                                                                                                        \
+    if (dtypes & GACT_DTYPES_F32) {                                                                           \
+      GACT_LAUNCH_QB(float, 1, M); GACT_LAUNCH_QB(float, 2, M); GACT_LAUNCH_QB(float, 4, M);                  \
+      GACT_LAUNCH_QB(float, 8, M);                                                                            \
+    }                                                                                                         \
+    if (dtypes & GACT_DTYPES_F16) {                                                                           \
+      GACT_LAUNCH_QB(f16, 1, M); GACT_LAUNCH_QB(f16, 2, M); GACT_LAUNCH_QB(f16, 4, M);                        \
+      GACT_LAUNCH_QB(f16, 8, M);                                                                              \
+    }                                                                                                         \
+  } while (0)
   switch (noise_mode) {
     case GACT_NOISE_CONST: GACT_LAUNCH_QB_ALL(GACT_NOISE_CONST); break;
     case GACT_NOISE_REF: GACT_LAUNCH_QB_ALL(GACT_NOISE_REF); break;

@@ -57,6 +57,10 @@ class BatchedQuantizer:
         self.device = torch.device(device)
         self.numels = [int(n) for n in numels]
         self.dtypes = list(dtypes)
+        # which element types occur (bit 0 float, bit 1 half): the library launches only their kernels
+        self.dtype_mask = 0
+        for dt in self.dtypes:
+            self.dtype_mask |= 1 << _abi.dtype_code(dt)
         self.L = len(self.numels)
         self.first_blocks, self.stats_offsets = [], []
         blocks = 0
@@ -128,7 +132,8 @@ class BatchedQuantizer:
             _abi.check(lib.gact_batch_plan(table.data_ptr(), bits.data_ptr(), self.L, packed.numel(),
                                            plan.data_ptr(), st))
             _abi.check(lib.gact_quantize_batched(table.data_ptr(), bits.data_ptr(), self.L, self.total_blocks, mode,
-                                                 plan.data_ptr(), self.block_map.data_ptr(), packed.data_ptr(),
+                                                 self.dtype_mask, plan.data_ptr(), self.block_map.data_ptr(),
+                                                 packed.data_ptr(),
                                                  scale.data_ptr(), mn.data_ptr(), st))
         # the widths are kept as they were at quantize time: the caller may refresh its own copy
         return BatchedPacked(self, packed, scale, mn, table, bits.clone(), plan, [t.shape for t in tensors],

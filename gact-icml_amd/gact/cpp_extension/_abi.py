@@ -15,7 +15,7 @@ F32, F16 = 0, 1
 NOISE_CONST, NOISE_INJECT, NOISE_REF, NOISE_FAST = 0, 1, 2, 3
 NOISE_MODES = {"deterministic": NOISE_CONST, "inject": NOISE_INJECT, "reference": NOISE_REF, "fast": NOISE_FAST}
 GROUP = 256
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class BatchEntry(ctypes.Structure):
@@ -50,7 +50,7 @@ SIGNATURES = {
     "gact_calc_precision": (_i32, [_vp, _vp, _vp, _i64, _f64]),
     "gact_calc_precision_device": (_i32, [_vp, _vp, _vp, _i64, _f64, _vp, _vp]),
     "gact_batch_plan": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp]),
-    "gact_quantize_batched": (_i32, [_vp, _vp, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "gact_quantize_batched": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),
     "gact_dequantize_batched": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
 }
 

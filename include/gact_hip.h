@@ -17,7 +17,7 @@
 extern "C" {
 #endif
 
-#define GACT_ABI_VERSION 1
+#define GACT_ABI_VERSION 2
 
 /* element types of activations, min, max and scale */
 #define GACT_F32 0
@@ -118,10 +118,16 @@ int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int
  * the rows stay 32-byte aligned).  `block_map` (device int32[total_blocks], may be null) names the
  * tensor of every block; without it each block searches the table.  Results equal a loop of
  * gact_quantize / gact_dequantize over the tensors (gact/gact/quantizer.py:95-142 drives the reference
- * one tensor at a time).  `plan` is the array gact_batch_plan filled. */
+ * one tensor at a time).  `plan` is the array gact_batch_plan filled.  `dtypes` says which element types
+ * occur in the table, which the host that built it knows: bit 0 float, bit 1 half (GACT_DTYPES_*); quantize
+ * launches only the kernels of those types (a half-only kernel needs a third fewer registers than one that
+ * also carries the float path), so a tensor whose type is missing from the mask is left unquantized. */
+#define GACT_DTYPES_F32 1
+#define GACT_DTYPES_F16 2
+#define GACT_DTYPES_ALL 3
 int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
-                          int noise_mode, const int64_t* plan, const int32_t* block_map, void* packed_arena,
-                          void* scale_arena, void* min_arena, void* stream);
+                          int noise_mode, int dtypes, const int64_t* plan, const int32_t* block_map,
+                          void* packed_arena, void* scale_arena, void* min_arena, void* stream);
 int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L,
                             int64_t total_blocks, const int64_t* plan, const int32_t* block_map,
                             const void* packed_arena, const void* scale_arena, const void* min_arena,
