@@ -1,5 +1,12 @@
-"""Adaptive per-tensor widths: estimate each saved tensor's sensitivity from gradient differences, then
-allocate widths greedily under an average-bits budget.  Mirrors gact/gact/autoprec.py of the reference."""
+"""Adaptive per-tensor widths.
+
+Every `adapt_interval` iterations the sensitivity of each saved tensor is measured from how much the
+parameter gradient moves when only that tensor is quantized differently (1 bit with two seeds, and 8 bit);
+the widths are then allocated greedily under the budget `avg_bits * total elements` by calc_precision.
+Same constructor, attributes and call order as gact/gact/autoprec.py of the reference, whose numbers
+(three probes per tensor, max(d01, 2 max(d02, d12)), the 1e10 cap, the variance warning) are kept.
+"""
+import contextlib
 import os
 import random
 
@@ -10,162 +17,171 @@ import torch.nn as nn
 from .cpp_extension import calc_precision as ext_calc_precision
 from .utils import exp_recorder
 
+SENSITIVITY_CAP = 1e10
+
+
+def _seed_everything(seed):
+    random.seed(seed)
+    np.random.seed(seed)
+    torch.manual_seed(seed)
+    if torch.cuda.is_available():
+        torch.cuda.manual_seed_all(seed)
+
+
+@contextlib.contextmanager
+def _probe_context(model, seed):
+    """An extra forward/backward must not move batch-norm running statistics nor the caller's CPU random
+    stream, and must itself be reproducible: fixed seed inside, state restored afterwards
+    (gact/gact/autoprec.py:80-100)."""
+    kinds = (nn.BatchNorm1d, nn.BatchNorm2d, nn.BatchNorm3d)
+    norms = [m for m in model.modules() if isinstance(m, kinds)] if model is not None else []
+    for m in norms:
+        m.track_running_stats = False
+    cpu_state = torch.get_rng_state().clone()
+    _seed_everything(seed)
+    try:
+        yield
+    finally:
+        torch.set_rng_state(cpu_state)
+        for m in norms:
+            m.track_running_stats = True
+
+
+def _sq_dist(a, b):
+    return ((a - b) ** 2).sum()
+
 
 class AutoPrecision:
     def __init__(self, model, quantizer, bits, max_bits, work_dir, adapt_interval, log_interval,
                  momentum=0.99, warmup_iter=100, debug=False):
-        self.model = model
-        self.quantizer = quantizer
-        self.debug = debug
+        self.model, self.quantizer = model, quantizer
+        self.avg_bits, self.max_bits = bits, max_bits
+        self.adapt_interval, self.log_iter = adapt_interval, log_interval
+        self.work_dir, self.debug = work_dir, debug
+        self.iter = 0
 
-        self.dims = None
-        self.bits = {}   # width per tensor id
-        self.C = {}      # sensitivity per tensor id
+        self.dims = None     # tensor id -> element count (the quantizer's table, adopted on first use)
+        self.bits = {}       # tensor id -> width
+        self.C = {}          # tensor id -> sensitivity
 
-        self.avg_bits = bits
-        self.max_bits = max_bits
-
-        # running estimate of the gradient variance, used for the "variance too large" warning
+        # exponential averages behind the "quantization variance is too large" warning
         self.momentum = momentum
         self.warmpup_iter = warmup_iter
         self.beta1 = 1e-7
         self.batch_grad = 0
         self.grad_var = 0
-        self.adapt_interval = adapt_interval
 
-        self.iter = 0
-        self.log_iter = log_interval
-        self.work_dir = work_dir
-
+    # ------------------------------------------------------------------ set-up
     def init_from_dims(self):
-        """gact/gact/autoprec.py:39-46."""
+        """Adopt the element counts the quantizer recorded on its first iteration; every tensor starts at
+        the average width with sensitivity 1 (gact/gact/autoprec.py:39-46)."""
         self.dims = self.quantizer.dims
-        total_ele = 0
-        for l in self.dims:
-            self.C[l] = 1.0
-            self.bits[l] = self.avg_bits
-            total_ele += self.dims[l]
-        self.total_bits = self.avg_bits * total_ele
+        self.C = {l: 1.0 for l in self.dims}
+        self.bits = {l: self.avg_bits for l in self.dims}
+        self.total_bits = self.avg_bits * sum(self.dims.values())
 
     def iterate_wrapper(self, backprop):
         if self.dims is None:
             self.init_from_dims()
         self.iterate(backprop)
 
-    # ---- helpers of iterate() ----
-    def _sample_grad(self):
-        return torch.cat([p.grad.ravel() for p in self.model.parameters() if p.grad is not None], 0)
-
-    @staticmethod
-    def _setup_seed(seed):
-        random.seed(seed)
-        np.random.seed(seed)
-        torch.manual_seed(seed)
-        if torch.cuda.is_available():
-            torch.cuda.manual_seed_all(seed)
-
-    @staticmethod
-    def _batch_norms(model):
-        return [m for m in model.modules() if isinstance(m, (nn.BatchNorm1d, nn.BatchNorm2d, nn.BatchNorm3d))]
-
+    # ------------------------------------------------------------------ probes
     def _get_grad(self, backprop):
-        """One extra forward + backward under a fixed seed, leaving running statistics and the global RNG
-        untouched.  gact/gact/autoprec.py:80-100."""
-        bns = self._batch_norms(self.model)
-        for bn in bns:
-            bn.track_running_stats = False
-        state = torch.get_rng_state().clone()
-        self._setup_seed(self.iter)
-        backprop()
-        torch.set_rng_state(state)
-        for bn in bns:
-            bn.track_running_stats = True
-        grad = self._sample_grad()
+        """Flattened parameter gradient of one extra pass; the quantizer's per-iteration state is reset after."""
+        with _probe_context(self.model, self.iter):
+            backprop()
+        flat = [p.grad.ravel() for p in self.model.parameters() if p.grad is not None]
         self.quantizer.iterate()
-        return grad
+        return torch.cat(flat, 0)
 
+    def _sensitivity_of(self, l, backprop):
+        """Three passes with only tensor l changed: 1 bit, 1 bit under the next seed, 8 bit."""
+        q = self.quantizer
+        kept = q.bits[l]
+        try:
+            q.bits[l] = 1
+            g_a = self._get_grad(backprop)
+            q.seeds[l] += 1
+            g_b = self._get_grad(backprop)
+            q.seeds[l] -= 1
+            q.bits[l] = 8
+            g_c = self._get_grad(backprop)
+        finally:
+            q.bits[l] = kept
+        sens = max(_sq_dist(g_a, g_b), 2 * max(_sq_dist(g_a, g_c), _sq_dist(g_b, g_c)))
+        if not torch.isfinite(sens) or sens > SENSITIVITY_CAP:
+            return SENSITIVITY_CAP
+        return sens.item()
+
+    def _predicted_variance(self, shift):
+        C = np.array([self.C[l] for l in self.C])
+        b = np.array([self.bits[l] for l in self.C])
+        return (C * 2 ** (-2.0 * (b - shift))).sum()
+
+    def _record_state(self, **extra):
+        exp_recorder.record("iter", self.iter)
+        exp_recorder.record("layer sensitivity", self.C)
+        exp_recorder.record("bits", self.bits)
+        exp_recorder.record("dims", self.dims)
+        for k, v in extra.items():
+            exp_recorder.record(k, v)
+        os.makedirs(self.work_dir, exist_ok=True)
+        exp_recorder.dump(os.path.join(self.work_dir, "autoprec.log"))
+
+    # ------------------------------------------------------------------ per iteration
     def iterate(self, backprop):
         """gact/gact/autoprec.py:57-186."""
-        if self.iter % self.adapt_interval == 0:
+        adapting = self.iter % self.adapt_interval == 0
+        if adapting:
             print('GACT: Initializing AutoPrec..., run extra %d iters' % (len(self.quantizer.bits)))
-            for l in self.quantizer.bits:
-                b = self.quantizer.bits[l]
-                # the same tensor at 1 bit with two seeds, and at 8 bits
-                self.quantizer.bits[l] = 1
-                grad0 = self._get_grad(backprop)
-                self.quantizer.seeds[l] += 1
-                grad1 = self._get_grad(backprop)
-                self.quantizer.seeds[l] -= 1
-                self.quantizer.bits[l] = 8
-                grad2 = self._get_grad(backprop)
-                diff01 = ((grad0 - grad1) ** 2).sum()
-                diff02 = ((grad0 - grad2) ** 2).sum()
-                diff12 = ((grad1 - grad2) ** 2).sum()
-                sens = max(diff01, max(diff02, diff12) * 2)
-                del grad0, grad1, grad2
-                if torch.isnan(sens) or torch.isinf(sens) or sens > 1e10:
-                    self.C[l] = 1e10
-                else:
-                    self.C[l] = sens.item()
-                self.quantizer.bits[l] = b
+            for l in list(self.quantizer.bits):
+                self.C[l] = self._sensitivity_of(l, backprop)
             self.refresh_bits()
 
-        if self.debug and self.iter % self.adapt_interval == 0:
-            grad = self._get_grad(backprop)
-            saved = dict(self.quantizer.bits)
-            for l in self.quantizer.bits:
-                self.quantizer.bits[l] = 32
-            det_grad = self._get_grad(backprop)
-            ap_var = ((grad - det_grad) ** 2).sum()
-            predicted = (np.array([self.C[l] for l in self.C]) *
-                         2 ** (-2.0 * (np.array([self.bits[l] for l in self.C]) - 1))).sum()
-            print('Exact Variance %f, Predicted Variance %f' % (ap_var.item(), predicted.item()))
-            self.quantizer.bits = saved
+        if adapting and self.debug:
+            # the variance model against a measurement: gradient at the allocated widths vs uncompressed
+            noisy = self._get_grad(backprop)
+            allocated = dict(self.quantizer.bits)
+            self.quantizer.bits = {l: 32 for l in allocated}
+            exact = self._get_grad(backprop)
+            print('Exact Variance %f, Predicted Variance %f'
+                  % (_sq_dist(noisy, exact).item(), self._predicted_variance(1).item()))
+            for b in (4,):
+                self.quantizer.bits = {l: b for l in allocated}
+                uniform = self._get_grad(backprop)
+                model_var = (np.array(list(self.C.values())) * 2 ** (-2.0 * (b - 1))).sum()
+                print('use %d bit to compare, exact variance %f, predicted variance %f'
+                      % (b, _sq_dist(uniform, exact).item(), model_var.item()))
+            self.quantizer.bits = self.bits.copy()
 
         if self.log_iter > 0 and self.iter % self.log_iter == 0:
-            det_grad = self._get_grad(backprop)
+            g = self._get_grad(backprop)
             m = self.momentum
             self.beta1 = self.beta1 * m + 1 - m
-            self.batch_grad = self.batch_grad * m + (1 - m) * det_grad
-            bgrad = self.batch_grad / self.beta1
-            gvar = ((bgrad - det_grad) ** 2).sum()
-            self.grad_var = self.grad_var * m + (1 - m) * gvar
-            exp_recorder.record("iter", self.iter)
-            exp_recorder.record("layer sensitivity", self.C)
-            exp_recorder.record("bits", self.bits)
-            exp_recorder.record("dims", self.dims)
-            os.makedirs(self.work_dir, exist_ok=True)
-            exp_recorder.dump(os.path.join(self.work_dir, "autoprec.log"))
+            self.batch_grad = self.batch_grad * m + (1 - m) * g
+            self.grad_var = self.grad_var * m + (1 - m) * _sq_dist(self.batch_grad / self.beta1, g)
+            self._record_state()
 
         self.iter += 1
 
     def refresh_bits(self):
-        """Greedy allocation from the current sensitivities.  gact/gact/autoprec.py:188-209: every tensor
-        starts at max_bits, the budget is avg_bits * total elements."""
-        l_list = list(self.dims)
-        dims_list = [self.dims[l] for l in l_list]
-        C_list = [self.C[l] for l in l_list]
-
-        bits_tensor = torch.ones(len(self.bits), dtype=torch.int32) * self.max_bits
-        bits_tensor = ext_calc_precision.calc_precision(bits_tensor, torch.tensor(C_list, dtype=torch.float),
-                                                        torch.tensor(dims_list, dtype=torch.int64), self.total_bits)
-        for i, l in enumerate(l_list):
-            self.bits[l] = bits_tensor[i].item()
+        """Greedy allocation from the current sensitivities: every tensor starts at max_bits, tensors are
+        listed in the order of the dims table (gact/gact/autoprec.py:188-209)."""
+        order = list(self.dims)
+        start = torch.full((len(self.bits),), self.max_bits, dtype=torch.int32)
+        chosen = ext_calc_precision.calc_precision(start,
+                                                   torch.tensor([self.C[l] for l in order], dtype=torch.float),
+                                                   torch.tensor([self.dims[l] for l in order], dtype=torch.int64),
+                                                   self.total_bits)
+        for l, b in zip(order, chosen.tolist()):
+            self.bits[l] = b
         self.quantizer.bits = self.bits.copy()
 
         if self.log_iter > 0 and self.iter > self.warmpup_iter:
             overall_var = self.grad_var / self.beta1
-            quantization_var = (np.array([self.C[l] for l in self.C]) *
-                                2 ** (-2.0 * np.array([self.bits[l] for l in self.C]))).sum()
+            quantization_var = self._predicted_variance(0)
             if quantization_var > overall_var * 0.1:
                 print('GACT Warning: Quantization variance is too large. Consider increasing number of bits.',
                       quantization_var, overall_var)
-                exp_recorder.record("iter", self.iter)
-                exp_recorder.record("layer sensitivity", self.C)
-                exp_recorder.record("bits", self.bits)
-                exp_recorder.record("dims", self.dims)
-                exp_recorder.record("warning", True)
-                exp_recorder.record("quantization var", float(quantization_var))
-                exp_recorder.record("overall var", float(overall_var))
-                os.makedirs(self.work_dir, exist_ok=True)
-                exp_recorder.dump(os.path.join(self.work_dir, "autoprec.log"))
+                self._record_state(**{"warning": True, "quantization var": float(quantization_var),
+                                      "overall var": float(overall_var)})

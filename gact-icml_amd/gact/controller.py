@@ -1,39 +1,67 @@
-"""User-facing driver: installs the saved-tensor hooks and advances the per-iteration state.
-Mirrors gact/gact/controller.py of the reference (same constructor, same methods)."""
+"""The object a training script holds: it installs the saved-tensor hooks and advances the per-iteration
+state of the quantizer and of auto precision.  Same constructor and methods as gact/gact/controller.py of
+the reference; also usable as a context manager (`with Controller(model) as c:` installs and removes the
+hooks).
+"""
+import bisect
+
 import torch
 
 from .autoprec import AutoPrecision
 from .conf import config
 from .quantizer import Quantizer
 
+_hooks = torch._C._autograd
+
 
 def default_bit_for(bit):
-    """Width used before auto precision has run: 2 stays 2, up to 4 -> 4, anything wider -> 8
-    (gact/gact/controller.py:13-23)."""
+    """Width used until auto precision has allocated widths: the next of 2, 4, 8 at or above the average
+    (gact/gact/controller.py:13-23: 2 -> 2, 3..4 -> 4, 5..16 -> 8)."""
     assert 1 < bit <= 16
-    if bit == 2:
-        return 2
-    if bit <= 4:
-        return 4
-    return 8
+    steps = (2, 4, 8)
+    return steps[min(bisect.bisect_left(steps, bit), 2)]
+
+
+def _to_pinned_host(t):
+    host = torch.empty(t.shape, dtype=t.dtype, device='cpu', pin_memory=True)
+    host.copy_(t, non_blocking=True)
+    return host
 
 
 class Controller:
     def __init__(self, model):
+        self._hooked = False
         if not config.compress_activation:
-            return
+            return      # hooks still work: they pass tensors through (or swap them when config.swap is set)
         self.model = model
-        self.quantizer = Quantizer(default_bit=default_bit_for(config.bit), swap=config.swap,
-                                   prefetch=config.prefetch)
-        self.quantizer.filter_tensors(model.named_parameters())   # parameters are never compressed
-
-        self.auto_prec = config.auto_prec
-        if self.auto_prec:
-            self.ap = AutoPrecision(self.model, self.quantizer, config.bit, config.max_bit, config.work_dir,
-                                    config.adapt_interval, config.log_interval)
         self.bit = config.bit
         self.iter = 0
-        self._hooked = False
+        self.quantizer = Quantizer(default_bit=default_bit_for(config.bit), swap=config.swap,
+                                   prefetch=config.prefetch)
+        # parameters are saved for backward too, and must stay exact
+        self.quantizer.filter_tensors(model.named_parameters())
+        self.auto_prec = config.auto_prec
+        if self.auto_prec:
+            self.ap = AutoPrecision(model, self.quantizer, config.bit, config.max_bit, config.work_dir,
+                                    config.adapt_interval, config.log_interval)
+
+    # ---- hooks (controller.py:53-60 of the reference: the default saved-tensor hooks of autograd) ----
+    def install_hook(self):
+        _hooks._push_saved_tensors_default_hooks(self.quantize, self.dequantize)
+        self._hooked = True
+
+    def uninstall_hook(self):
+        if getattr(self, "_hooked", False):
+            _hooks._pop_saved_tensors_default_hooks()
+            self._hooked = False
+
+    def __enter__(self):
+        self.install_hook()
+        return self
+
+    def __exit__(self, *exc):
+        self.uninstall_hook()
+        return False
 
     def __del__(self):
         try:
@@ -41,24 +69,22 @@ class Controller:
         except Exception:
             pass
 
-    def install_hook(self):
-        def pack_hook(x):
-            return self.quantize(x)
+    # ---- what the hooks do ----
+    def quantize(self, input):
+        if config.compress_activation:
+            return self.quantizer.quantize(input)
+        return _to_pinned_host(input) if config.swap else input
 
-        def unpack_hook(x):
-            return self.dequantize(x)
+    def dequantize(self, input):
+        if config.compress_activation:
+            return self.quantizer.dequantize(input)
+        return input.cuda(non_blocking=True) if config.swap else input
 
-        torch._C._autograd._push_saved_tensors_default_hooks(pack_hook, unpack_hook)
-        self._hooked = True
-
-    def uninstall_hook(self):
-        if getattr(self, "_hooked", False):
-            torch._C._autograd._pop_saved_tensors_default_hooks()
-            self._hooked = False
-
+    # ---- once per training iteration, after the optimizer step ----
     def iterate(self, get_grad):
-        """Call once per training iteration, after the optimizer step.  `get_grad` runs one forward +
-        backward pass; auto precision calls it when it refreshes the sensitivities."""
+        """`get_grad` runs one forward + backward pass; auto precision calls it when it re-measures the
+        sensitivities.  Order as in controller.py:74-78: reset the quantizer, let auto precision run, then
+        move the seed offset to the new iteration."""
         if not config.compress_activation:
             return
         self.quantizer.iterate()
@@ -66,19 +92,3 @@ class Controller:
             self.ap.iterate_wrapper(get_grad)
         self.iter += 1
         self.quantizer.seed_iter = self.iter
-
-    def quantize(self, input):
-        if not config.compress_activation:
-            if config.swap:
-                host = torch.empty(input.shape, dtype=input.dtype, device='cpu', pin_memory=True)
-                host.copy_(input, non_blocking=True)
-                return host
-            return input
-        return self.quantizer.quantize(input)
-
-    def dequantize(self, input):
-        if not config.compress_activation:
-            if config.swap:
-                input = input.cuda(non_blocking=True)
-            return input
-        return self.quantizer.dequantize(input)

@@ -1,67 +1,110 @@
-"""Small helpers used by the quantizer and the auto-precision driver (gact/gact/utils.py of the reference)."""
+"""Helpers next to the compression path, with the names of gact/gact/utils.py of the reference: tensor
+keys for duplicate detection, memory accounting, and the JSON-lines recorder auto precision logs to."""
+import collections
 import json
-from collections import OrderedDict
+import math
 
 import numpy as np
 import torch
 
+# ---------------------------------------------------------------- tensor keys (utils.py:6-38 of the reference)
+
+
+def _key_prefix(t, add_dataptr):
+    return [t.data_ptr()] if add_dataptr else []
+
 
 def uniform_sample(input, sample_cnt, add_dataptr=True):
-    """Evenly spaced sample of a tensor's values (optionally prefixed by its address): the key that
-    recognises a tensor saved twice.  gact/gact/utils.py:16-24."""
-    num_elem = input.numel()
-    sample_cnt = min(num_elem, sample_cnt)
-    key = [input.data_ptr()] if add_dataptr else []
-    if sample_cnt > 0:
-        idx = torch.arange(0, sample_cnt, dtype=torch.long, device=input.device) * (num_elem // sample_cnt)
-        key += input.ravel()[idx].tolist()
-    return key
+    """Key of a tensor: (its address and) min(sample_cnt, numel) values taken at a constant stride.  Two saved
+    tensors with the same key are treated as the same tensor.  One gather on the tensor's device instead of
+    one host read per value."""
+    n = input.numel()
+    take = min(n, sample_cnt)
+    if take == 0:
+        return _key_prefix(input, add_dataptr)
+    positions = torch.arange(take, device=input.device) * (n // take)
+    return _key_prefix(input, add_dataptr) + input.ravel()[positions].tolist()
+
+
+def uniform_sample_ref(input, sample_cnt, add_dataptr=True):
+    """The same key read value by value; what uniform_sample is tested against."""
+    stride = max(input.numel() // sample_cnt, 1)
+    flat = input.reshape(-1)
+    return _key_prefix(input, add_dataptr) + [flat[i * stride].item() for i in range(min(sample_cnt, input.numel()))]
+
+
+def random_sample(input, sample_cnt, add_dataptr=True):
+    """Key from sample_cnt positions drawn with a generator seeded by the tensor's rank; the global random
+    state is left as it was."""
+    saved = torch.get_rng_state()
+    torch.manual_seed(input.dim())
+    positions = torch.randint(0, input.numel(), (sample_cnt,))
+    torch.set_rng_state(saved)
+    return _key_prefix(input, add_dataptr) + input.reshape(-1)[positions.to(input.device)].tolist()
+
+
+# ---------------------------------------------------------------- memory accounting (utils.py:40-78)
+
+_MB = 1024.0 * 1024.0
 
 
 def get_memory_usage(print_info=False):
-    """Bytes currently allocated by torch on the GPU.  gact/gact/utils.py:40-47."""
+    """Bytes torch has allocated on the current GPU."""
     allocated = torch.cuda.memory_allocated()
     if print_info:
-        print("allocated: %.2f MB" % (allocated / 1024 / 1024), flush=True)
-        print("reserved:  %.2f MB" % (torch.cuda.memory_reserved() / 1024 / 1024), flush=True)
+        print("allocated: %.2f MB" % (allocated / _MB), flush=True)
+        print("reserved:  %.2f MB" % (torch.cuda.memory_reserved() / _MB), flush=True)
     return allocated
 
 
-_ELEM_BYTES = {torch.long: 8, torch.float32: 4, torch.int: 4, torch.bfloat16: 2, torch.float16: 2, torch.int16: 2,
-               torch.int8: 1, torch.uint8: 1}
+_COUNTED_DTYPES = (torch.long, torch.float32, torch.int, torch.bfloat16, torch.float16, torch.int16, torch.int8,
+                   torch.uint8)
 
 
 def compute_tensor_bytes(tensors):
-    """Bytes held by a tensor or a list of tensors / ints.  gact/gact/utils.py:49-70."""
-    if not isinstance(tensors, (list, tuple)):
-        tensors = [tensors]
+    """Bytes held by a tensor or a list of tensors; a plain int in the list counts 4 bytes.  The dtypes the
+    reference counts are accepted, anything else is an error."""
+    items = tensors if isinstance(tensors, (list, tuple)) else [tensors]
     total = 0
-    for x in tensors:
+    for x in items:
         if type(x) == int:
             total += 4
-        elif x.dtype in _ELEM_BYTES:
-            total += int(np.prod(x.size())) * _ELEM_BYTES[x.dtype]
+        elif x.dtype in _COUNTED_DTYPES:
+            total += math.prod(x.size()) * x.element_size()
         else:
             raise TypeError("unsupported dtype %s" % x.dtype)
     return total
 
 
+def empty_cache(ratio):
+    """Return cached blocks to the driver when less than `ratio` of the reserved memory is in use."""
+    if ratio is None:
+        return
+    reserved = torch.cuda.memory_reserved(0)
+    if reserved > 0 and torch.cuda.memory_allocated(0) / reserved < ratio:
+        torch.cuda.empty_cache()
+
+
+# ---------------------------------------------------------------- experiment log (utils.py:80-101)
+
+
 class GlobalExpRecorder:
-    """Key/value record appended to a file as one JSON line per dump.  gact/gact/utils.py:80-101."""
+    """Latest value per key; dump() appends them to a file as one JSON line."""
 
     def __init__(self):
-        self.val_dict = OrderedDict()
+        self.val_dict = collections.OrderedDict()
 
     def record(self, key, value, float_round=6):
-        if isinstance(value, (np.int32, np.int64)):
+        if isinstance(value, np.integer):
             value = int(value)
-        if isinstance(value, (float, np.float32, np.float64)):
+        elif isinstance(value, (float, np.floating)):
             value = round(float(value), float_round)
         self.val_dict[key] = value
 
     def dump(self, filename):
-        with open(filename, "a") as fout:
-            fout.write(json.dumps(self.val_dict) + '\n')
+        with open(filename, "a") as out:
+            out.write(json.dumps(self.val_dict))
+            out.write("\n")
 
     def clear(self):
         pass

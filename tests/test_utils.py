@@ -4,7 +4,8 @@ import json
 
 import torch
 
-from gact.utils import GlobalExpRecorder, compute_tensor_bytes, uniform_sample
+from gact.utils import (GlobalExpRecorder, compute_tensor_bytes, empty_cache, random_sample, uniform_sample,
+                        uniform_sample_ref)
 
 
 def sample_by_loop(t, cnt, add_dataptr=True):
@@ -21,7 +22,23 @@ def test_uniform_sample_matches_a_plain_loop():
         t = torch.randn(shape)
         assert uniform_sample(t, cnt) == sample_by_loop(t, cnt)
         assert uniform_sample(t, cnt, add_dataptr=False) == sample_by_loop(t, cnt, add_dataptr=False)
+        assert uniform_sample(t, cnt) == uniform_sample_ref(t, cnt)
     assert uniform_sample(torch.empty(0), 10, add_dataptr=False) == []
+
+
+def test_random_sample_is_reproducible_and_leaves_the_global_stream_alone():
+    t = torch.arange(1000.0).reshape(10, 100)
+    torch.manual_seed(5)
+    before = torch.rand(3)
+    torch.manual_seed(5)
+    key = random_sample(t, 20)
+    after = torch.rand(3)
+    assert torch.equal(before, after)
+    assert key[0] == t.data_ptr() and len(key) == 21
+    assert key == random_sample(t, 20) and all(0 <= v < 1000 for v in key[1:])
+    g = torch.Generator().manual_seed(t.dim())          # the positions come from a generator seeded by the rank
+    assert key[1:] == t.reshape(-1)[torch.randint(0, 1000, (20,), generator=g)].tolist()
+    empty_cache(None)                                    # no ratio: nothing to do, no GPU needed
 
 
 def test_compute_tensor_bytes():
