@@ -62,6 +62,32 @@ def test_pack_unpack_entry_points(dtype, bits, ngd, stream):
     np.testing.assert_array_equal(bits_view(out.cpu().numpy().reshape(-1)), bits_view(ref.reshape(-1)))
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f16"])
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("ngd", [(67, 1, 256), (13, 2, 96)])
+def test_pack_with_min_max_narrower_than_the_data(dtype, bits, ngd):
+    """Caller-supplied min / max that do not bracket the data: elements below min give negative products
+    (code 0), elements above max give codes beyond 2^bits - 1 whose shifted bits spill into the neighbouring
+    fields or fall off the byte (quantization_cuda_kernel.cu:66-67).  All of it must match the restatement."""
+    N, G, D = ngd
+    g = torch.Generator().manual_seed(100 + bits)
+    x = torch.randn((N, G, D), generator=g).to(dtype)
+    mn_np = np.full(N * G, -0.5, dtype=x.numpy().dtype) + (np.arange(N * G) % 5).astype(x.numpy().dtype) * 0.1
+    mx_np = mn_np + np.asarray(0.7, dtype=mn_np.dtype)
+    sc_np = oracle.scale(mn_np, mx_np, bits)
+    xd = x.cuda()
+    mn = torch.from_numpy(mn_np).reshape(N, G, 1).cuda()
+    mx = torch.from_numpy(mx_np).reshape(N, G, 1).cuda()
+    for stream, mode in (("deterministic", 0), ("reference", 2), ("fast", 3)):
+        want = oracle.pack(x.numpy(), mn_np, sc_np, bits, mode, 23)
+        packed, scale = ext_quantization.pack_single_precision(xd, mn, mx, bits, True, 23, rng_stream=stream)
+        np.testing.assert_array_equal(bits_view(scale.cpu().numpy().reshape(-1)), bits_view(sc_np))
+        np.testing.assert_array_equal(packed.cpu().numpy().view(np.uint8)[:want.size], want)
+        out = ext_quantization.unpack_single_precision(packed, bits, scale, mn, N, G, D)
+        ref = oracle.unpack(want, bits, sc_np, mn_np, N, G, D)
+        np.testing.assert_array_equal(bits_view(out.cpu().numpy().reshape(-1)), bits_view(ref.reshape(-1)))
+
+
 def test_pack_uses_the_min_max_it_is_given():
     # the entry point's contract: codes are taken against the caller's min / max, whatever the data holds
     x = torch.rand((16, 1, 256)) * 0.5 + 0.25
