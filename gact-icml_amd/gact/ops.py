@@ -19,9 +19,19 @@ def _num_groups(numel):
     return (numel + config.group_size - 1) // config.group_size
 
 
-def _require_group_256():
-    if config.group_size != _abi.GROUP:
-        raise RuntimeError("the fused kernels are built for group_size 256, got %d" % config.group_size)
+def _fused():
+    """The single-pass kernels are built for groups of 256; any other config.group_size takes the
+    extension-style sequence minimax -> pack / unpack on the zero-padded tensor, as the reference does."""
+    return config.group_size == _abi.GROUP
+
+
+def _padded_groups(input):
+    """gact/gact/ops.py:12-19: flatten, zero-pad to whole groups, [N, group_size]."""
+    group = config.group_size
+    pad = _num_groups(input.numel()) * group - input.numel()
+    if pad > 0:
+        input = torch.cat([input.reshape(1, -1), torch.zeros([1, pad], dtype=input.dtype, device=input.device)], dim=1)
+    return input.reshape(-1, group)
 
 
 def no_scheme_quantize_pack(input, q_bit, seed, *, noise=None, rng_stream=None):
@@ -29,17 +39,20 @@ def no_scheme_quantize_pack(input, q_bit, seed, *, noise=None, rng_stream=None):
     N = _num_groups(input.numel())
     if q_bit == 32:
         # the passthrough of ops.py:21-24: the padded [N, group] view itself, max - min, min
-        num_ele = N * config.group_size
-        pad_num = num_ele - input.numel()
-        if pad_num > 0:
-            input = torch.cat([input.reshape(1, -1),
-                               torch.zeros([1, pad_num], dtype=input.dtype, device=input.device)], dim=1)
-        input_groups = input.reshape(-1, config.group_size)
+        input_groups = _padded_groups(input)
         q_min = input_groups.min(dim=-1, keepdim=True).values
         q_scale = input_groups.max(dim=-1, keepdim=True).values - q_min
         return input_groups, q_scale, q_min
 
-    _require_group_256()
+    if not _fused():
+        from .cpp_extension import minimax as ext_minimax
+        input_groups = _padded_groups(input.contiguous()).contiguous()
+        q_min, mx = ext_minimax.minimax(input_groups)
+        q_input, q_scale = ext_quantization.pack_single_precision(
+            input_groups.view(N, 1, -1), q_min.view(N, 1, 1), mx.view(N, 1, 1), q_bit, True, seed,
+            noise=noise, rng_stream=rng_stream)
+        return q_input, q_scale, q_min.view(N, 1, 1)
+
     if not input.is_cuda:
         raise RuntimeError("data must be a CUDA tensor!")
     if input.dtype not in (torch.float32, torch.float16):
@@ -106,7 +119,10 @@ def op_dequantize(input, input_shape):
     if q_bit == 32:
         return q_input.ravel()[:num_features].reshape(*input_shape).contiguous()
 
-    _require_group_256()
+    if not _fused():
+        groups = dequantize_and_unpack(q_input, input_shape, q_bit, q_scale, q_min)
+        return groups.ravel()[:num_features].reshape(*input_shape).contiguous()
+
     ext_quantization._check_bits(q_bit)
     if not q_input.is_cuda:
         raise RuntimeError("data must be a CUDA tensor!")

@@ -288,3 +288,34 @@ def test_random_cases_against_the_oracle():
         except AssertionError as e:
             raise AssertionError("case %d: dtype %s bits %d stream %s numel %d seed %d: %s"
                                  % (case, x.dtype, bits, mode, x.numel(), seed, e))
+
+
+@pytest.mark.parametrize("group", [64, 128, 512])
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f16"])
+def test_other_group_sizes_take_the_extension_sequence(group, dtype):
+    """config.group_size other than 256 (gact/gact/conf.py:50 makes it a setting): zero-pad, minimax, pack,
+    unpack, slice - the reference's own sequence on the general-shape kernels."""
+    saved = config.group_size
+    config.group_size = group
+    try:
+        g = torch.Generator().manual_seed(group)
+        x_cpu = torch.randn((37, 101), generator=g).to(dtype)           # 3737 elements: a padded last group
+        N = -(-x_cpu.numel() // group)
+        flat = np.zeros(N * group, dtype=x_cpu.numpy().dtype)
+        flat[: x_cpu.numel()] = x_cpu.numpy().ravel()
+        groups = flat.reshape(N, group)
+        mn, mx = oracle.minimax(groups)
+        for bits in BITS:
+            sc = oracle.scale(mn, mx, bits)
+            for stream in ("deterministic", "fast", "reference"):
+                want = oracle.pack(groups.reshape(N, 1, group), mn, sc, bits, MODES[stream], 9)
+                q = ops.op_quantize(x_cpu.cuda(), bits, 9, rng_stream=stream)
+                assert q[0].numel() == want.size + 1 and q[2].shape == (N, 1, 1) and q[3].shape == (N, 1, 1)
+                np.testing.assert_array_equal(q[0].cpu().numpy().view(np.uint8)[: want.size], want)
+                np.testing.assert_array_equal(q[3].cpu().numpy().ravel(), mn)
+                out = ops.op_dequantize(q, x_cpu.shape)
+                ref = oracle.unpack(want, bits, sc, mn, N, 1, group).ravel()[: x_cpu.numel()].reshape(x_cpu.shape)
+                it = np.uint16 if ref.dtype == np.float16 else np.uint32
+                np.testing.assert_array_equal(out.cpu().numpy().view(it), ref.view(it))
+    finally:
+        config.group_size = saved
