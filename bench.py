@@ -302,7 +302,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS) + ["config5"])
     ap.add_argument("--all", action="store_true", help="also time the other single-tensor workloads (extra key)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -319,7 +319,12 @@ def main():
         sys.exit("bench.py needs a GPU")
     torch.cuda.set_device(0)
 
-    res, x = run_workload(torch, args.workload, args.steps, args.warmup)
+    if args.workload == "config5":
+        res, x = run_config5(torch, args.steps, args.warmup), None
+        res.update(bits="1/2/4/8 by calc_precision", dtype="float16")
+        args.copy_calibration, args.no_cpu = False, True     # no single tensor to copy or to hand to the CPU leg
+    else:
+        res, x = run_workload(torch, args.workload, args.steps, args.warmup)
     dom = "quantize" if res["quantize"]["ms"] >= res["dequantize"]["ms"] else "dequantize"
     achieved = res[dom]["gbs"]
     line = {
@@ -351,7 +356,8 @@ def main():
             r, _ = run_workload(torch, name, max(20, args.steps // 4), max(3, args.warmup // 4))
             extra.append(r)
             torch.cuda.empty_cache()
-        extra.append(run_config5(torch, 20, 3))
+        if args.workload != "config5":
+            extra.append(run_config5(torch, 20, 3))
         torch.cuda.empty_cache()
         line["other_workloads"] = extra
     if not args.no_cpu:
