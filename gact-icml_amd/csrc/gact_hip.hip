@@ -1332,26 +1332,45 @@ inline int quantize_threads(int bits, size_t elem_size) {
 }
 inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8 / bits); }
 
+// Fewer resident waves per CU for some float kernels on large tensors.  These streams mix a minority of
+// traffic in the other direction into their main direction, and past a point more requests in flight make
+// that mix more expensive for the memory system, not cheaper (a stand-alone kernel that writes 8 KB and reads
+// 1 KB per wave: 88 us for 411 MB at full occupancy, 70 us at 2 waves per SIMD).  The cap is a request for
+// dynamic LDS that the kernels never touch - a CU has 160 KB of it, so 53 000 bytes admit 3 workgroups.
+// Measured on a 411 MB float tensor, dequantize with 3 workgroups of 4 waves per CU: 1 bit 76 -> 65 us,
+// 2 bit 75 -> 70, 4 bit 80 -> 78, 8 bit 84 -> 79; quantize 1 bit with 8 one-wave workgroups 73 -> 69, 4 bit
+// with 16: 75.8 -> 73.4.  Half kernels and small tensors do not gain and keep full occupancy.
+constexpr int64_t kCapFromGroups = 1 << 16;  // 64 MB of float
+inline unsigned dequantize_lds_cap(size_t elem_size, int64_t N) {
+  return elem_size == 4 && N >= kCapFromGroups ? 53000u : 0u;
+}
+inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
+  if (elem_size != 4 || N < kCapFromGroups) return 0u;
+  return bits == 1 ? 20000u : bits == 4 ? 10000u : 0u;
+}
+
 template <typename T, int BITS, bool GIVEN>
 int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, T* scale, T* mn, T* mx, int noise_mode,
                     uint64_t seed, const float* noise, hipStream_t stream) {
   dim3 grid, block;
   row_grid(supergroups(N, BITS), &grid, &block, quantize_threads(BITS, sizeof(T)));
+  // the reference stream's one Philox block per byte makes the kernel instruction-bound: it wants every wave
+  const unsigned lds = noise_mode == GACT_NOISE_REF ? 0u : quantize_lds_cap(sizeof(T), BITS, N);
   switch (noise_mode) {
     case GACT_NOISE_CONST:
-      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_CONST, GIVEN>), grid, block, 0, stream, x, numel, N,
+      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_CONST, GIVEN>), grid, block, lds, stream, x, numel, N,
                          packed, scale, mn, mx, seed, noise);
       break;
     case GACT_NOISE_INJECT:
-      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_INJECT, GIVEN>), grid, block, 0, stream, x, numel, N,
+      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_INJECT, GIVEN>), grid, block, lds, stream, x, numel, N,
                          packed, scale, mn, mx, seed, noise);
       break;
     case GACT_NOISE_REF:
-      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_REF, GIVEN>), grid, block, 0, stream, x, numel, N,
+      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_REF, GIVEN>), grid, block, lds, stream, x, numel, N,
                          packed, scale, mn, mx, seed, noise);
       break;
     case GACT_NOISE_FAST:
-      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_FAST, GIVEN>), grid, block, 0, stream, x, numel, N,
+      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_FAST, GIVEN>), grid, block, lds, stream, x, numel, N,
                          packed, scale, mn, mx, seed, noise);
       break;
     default:
@@ -1378,12 +1397,13 @@ int dispatch_dequantize(int bits, const uint8_t* packed, const T* scale, const T
   // a unit of 8 groups takes 256 / (16 / sizeof(T)) lanes
   const int64_t units_per_block = 256 / (GROUP / (16 / (int64_t)sizeof(T)));
   const int64_t unit_groups = ROW_GROUPS;
+  const unsigned lds = dequantize_lds_cap(sizeof(T), N);
   const dim3 grid((unsigned)(((N + unit_groups - 1) / unit_groups + units_per_block - 1) / units_per_block)), block(256);
   switch (bits) {
-    case 1: hipLaunchKernelGGL((dequantize_kernel<T, 1>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
-    case 2: hipLaunchKernelGGL((dequantize_kernel<T, 2>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
-    case 4: hipLaunchKernelGGL((dequantize_kernel<T, 4>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
-    case 8: hipLaunchKernelGGL((dequantize_kernel<T, 8>), grid, block, 0, stream, packed, scale, mn, numel, N, out); break;
+    case 1: hipLaunchKernelGGL((dequantize_kernel<T, 1>), grid, block, lds, stream, packed, scale, mn, numel, N, out); break;
+    case 2: hipLaunchKernelGGL((dequantize_kernel<T, 2>), grid, block, lds, stream, packed, scale, mn, numel, N, out); break;
+    case 4: hipLaunchKernelGGL((dequantize_kernel<T, 4>), grid, block, lds, stream, packed, scale, mn, numel, N, out); break;
+    case 8: hipLaunchKernelGGL((dequantize_kernel<T, 8>), grid, block, lds, stream, packed, scale, mn, numel, N, out); break;
     default: return GACT_EINVAL;
   }
   return launch_status();
