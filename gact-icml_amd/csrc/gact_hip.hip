@@ -1338,15 +1338,15 @@ inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8
 // 1 KB per wave: 88 us for 411 MB at full occupancy, 70 us at 2 waves per SIMD).  The cap is a request for
 // dynamic LDS that the kernels never touch - a CU has 160 KB of it, so 53 000 bytes admit 3 workgroups.
 // Measured on a 411 MB float tensor, dequantize with 3 workgroups of 4 waves per CU: 1 bit 76 -> 65 us,
-// 2 bit 75 -> 70, 4 bit 80 -> 78, 8 bit 84 -> 79; quantize 1 bit with 8 one-wave workgroups 73 -> 69, 4 bit
-// with 16: 75.8 -> 73.4.  Half kernels and small tensors do not gain and keep full occupancy.
+// 2 bit 75 -> 70, 4 bit 80 -> 79, 8 bit 84 -> 79; quantize 1 bit with 8 one-wave workgroups 73 -> 69, 4 bit
+// with 13: 75.2 -> 74.0.  Half kernels and small tensors do not gain and keep full occupancy.
 constexpr int64_t kCapFromGroups = 1 << 16;  // 64 MB of float
 inline unsigned dequantize_lds_cap(size_t elem_size, int64_t N) {
   return elem_size == 4 && N >= kCapFromGroups ? 53000u : 0u;
 }
 inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
   if (elem_size != 4 || N < kCapFromGroups) return 0u;
-  return bits == 1 ? 20000u : bits == 4 ? 10000u : 0u;
+  return bits == 1 ? 20000u : bits == 4 ? 12000u : 0u;
 }
 
 template <typename T, int BITS, bool GIVEN>
