@@ -628,11 +628,26 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
     constexpr int ENT = 1 << BITS, GPP = 16 / ENT, PASSES = G / GPP;
     const float cf = (float)(rl & (ENT - 1));
     uint32_t tab[PASSES];
+    constexpr int PER16 = 16 / (int)sizeof(T);
+    if (GPP == 1 && G % PER16 == 0 && g0 + G <= N &&
+        ((reinterpret_cast<uintptr_t>(scale + g0) | reinterpret_cast<uintptr_t>(mn + g0)) & 15u) == 0) {
+      // one group per pass: every lane needs all 8 scales and minima, two 16-byte loads each instead of 16 small ones
+      typedef T vec16 __attribute__((ext_vector_type(PER16)));
+      vec16 sv[G / PER16], mv[G / PER16];
 #pragma unroll
-    for (int p = 0; p < PASSES; p++) {
-      const int64_t g = g0 + p * GPP + rl / ENT;
-      const bool live = g < N;
-      tab[p] = Elem<T>::table_entry(cf, live ? scale[g] : (T)1, live ? mn[g] : (T)0);
+      for (int c = 0; c < G / PER16; c++) {
+        sv[c] = *reinterpret_cast<const vec16*>(scale + g0 + c * PER16);
+        mv[c] = *reinterpret_cast<const vec16*>(mn + g0 + c * PER16);
+      }
+#pragma unroll
+      for (int p = 0; p < PASSES; p++) tab[p] = Elem<T>::table_entry(cf, sv[p / PER16][p % PER16], mv[p / PER16][p % PER16]);
+    } else {
+#pragma unroll
+      for (int p = 0; p < PASSES; p++) {
+        const int64_t g = g0 + p * GPP + rl / ENT;
+        const bool live = g < N;
+        tab[p] = Elem<T>::table_entry(cf, live ? scale[g] : (T)1, live ? mn[g] : (T)0);
+      }
     }
     const uint32_t rowbase = threadIdx.x & 48u;
 #pragma unroll
