@@ -1347,21 +1347,25 @@ inline int quantize_threads(int bits, size_t elem_size) {
 }
 inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8 / bits); }
 
-// Fewer resident waves per CU for some float kernels on large tensors.  These streams mix a minority of
-// traffic in the other direction into their main direction, and past a point more requests in flight make
-// that mix more expensive for the memory system, not cheaper (a stand-alone kernel that writes 8 KB and reads
-// 1 KB per wave: 88 us for 411 MB at full occupancy, 70 us at 2 waves per SIMD).  The cap is a request for
-// dynamic LDS that the kernels never touch - a CU has 160 KB of it, so 53 000 bytes admit 3 workgroups.
-// Measured on a 411 MB float tensor, dequantize with 3 workgroups of 4 waves per CU: 1 bit 76 -> 65 us,
-// 2 bit 75 -> 70, 4 bit 80 -> 79, 8 bit 84 -> 79; quantize 1 bit with 8 one-wave workgroups 73 -> 69, 4 bit
-// with 13: 75.2 -> 74.0.  Half kernels and small tensors do not gain and keep full occupancy.
-constexpr int64_t kCapFromGroups = 1 << 16;  // 64 MB of float
-inline unsigned dequantize_lds_cap(size_t elem_size, int64_t N) {
-  return elem_size == 4 && N >= kCapFromGroups ? 53000u : 0u;
+// Fewer resident waves per CU for some kernels on large tensors.  These streams mix a minority of traffic in
+// the other direction into their main direction, and past a point more requests in flight make that mix more
+// expensive for the memory system, not cheaper (a stand-alone kernel that writes 8 KB and reads 1 KB per
+// wave: 88 us for 411 MB at full occupancy, 70 us at 2 waves per SIMD).  The cap is a request for dynamic
+// LDS that the kernels never touch - a CU has 160 KB of it, so 53 000 bytes admit 3 workgroups.
+// Interleaved A/B on a 411 MB float tensor (us, full occupancy -> capped): dequantize with 3 workgroups of
+// 4 waves per CU 1 bit 77.0 -> 65.8, 2 bit 76.2 -> 70.1, 4 bit 80.7 -> 78.1, 8 bit 83.9 -> 80.1; half 8 bit
+// with 4 workgroups 66.4 -> 63.7; quantize float 2 bit with 10 one-wave workgroups 71.5 -> 69.5, 4 bit with
+// 16: 75.6 -> 72.8.  The other kernels (all half quantize, float quantize at 1 and 8 bit) and small tensors
+// gain nothing or lose, and keep full occupancy.
+constexpr int64_t kCapFromGroups = 1 << 16;  // 16.8 M elements
+inline unsigned dequantize_lds_cap(size_t elem_size, int bits, int64_t N) {
+  if (N < kCapFromGroups) return 0u;
+  if (elem_size == 4) return 53000u;
+  return bits == 8 ? 40000u : 0u;
 }
 inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
   if (elem_size != 4 || N < kCapFromGroups) return 0u;
-  return bits == 1 ? 20000u : bits == 4 ? 12000u : 0u;
+  return bits == 2 ? 16000u : bits == 4 ? 10000u : 0u;
 }
 
 template <typename T, int BITS, bool GIVEN>
@@ -1412,7 +1416,7 @@ int dispatch_dequantize(int bits, const uint8_t* packed, const T* scale, const T
   // a unit of 8 groups takes 256 / (16 / sizeof(T)) lanes
   const int64_t units_per_block = 256 / (GROUP / (16 / (int64_t)sizeof(T)));
   const int64_t unit_groups = ROW_GROUPS;
-  const unsigned lds = dequantize_lds_cap(sizeof(T), N);
+  const unsigned lds = dequantize_lds_cap(sizeof(T), bits, N);
   const dim3 grid((unsigned)(((N + unit_groups - 1) / unit_groups + units_per_block - 1) / units_per_block)), block(256);
   switch (bits) {
     case 1: hipLaunchKernelGGL((dequantize_kernel<T, 1>), grid, block, lds, stream, packed, scale, mn, numel, N, out); break;
