@@ -806,8 +806,11 @@ __host__ __device__ constexpr int dq_supergroups(int bits) { return ROW_GROUPS /
 #ifndef GACT_XCD_RUN_DQ
 #define GACT_XCD_RUN_DQ 16
 #endif
+#ifndef GACT_XCD_RUN_Q_LOW
+#define GACT_XCD_RUN_Q_LOW 0 /* quantize, 1 and 2 bit */
+#endif
 #ifndef GACT_XCD_RUN_Q
-#define GACT_XCD_RUN_Q 32 /* quantize, 4 and 8 bit (2-3 % there; the 1 and 2 bit kernels lose with it) */
+#define GACT_XCD_RUN_Q 128 /* quantize, 4 and 8 bit (2-4 % there; the 1 and 2 bit kernels gain nothing or lose) */
 #endif
 template <uint32_t RUN>
 __device__ __forceinline__ uint32_t xcd_tile(uint32_t b, uint32_t nb) {
@@ -823,7 +826,7 @@ template <typename T, int BITS, int NOISE, bool GIVEN>
 __global__ void __launch_bounds__(256)
 quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
                 T* __restrict__ scale_out, T* mn_io, T* mx_io, uint64_t seed, const float* __restrict__ noise) {
-  constexpr uint32_t RUN = BITS >= 4 ? GACT_XCD_RUN_Q : 0;
+  constexpr uint32_t RUN = BITS >= 4 ? GACT_XCD_RUN_Q : GACT_XCD_RUN_Q_LOW;
   const int64_t sg = (int64_t)xcd_tile<RUN>(blockIdx.x, gridDim.x) * (blockDim.x >> 4) + (threadIdx.x >> 4);
   if (sg * (8 / BITS) >= N) return;
   quantize_supergroup<T, BITS, NOISE, GIVEN>(x, numel, N, sg, threadIdx.x & 15, packed, scale_out, mn_io, mx_io,
