@@ -1355,11 +1355,11 @@ inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8
 // expensive for the memory system, not cheaper (a stand-alone kernel that writes 8 KB and reads 1 KB per
 // wave: 88 us for 411 MB at full occupancy, 70 us at 2 waves per SIMD).  The cap is a request for dynamic
 // LDS that the kernels never touch - a CU has 160 KB of it, so 53 000 bytes admit 3 workgroups.
-// Interleaved A/B on a 411 MB float tensor (us, full occupancy -> capped): dequantize with 3 workgroups of
-// 4 waves per CU 1 bit 77.0 -> 65.8, 2 bit 76.2 -> 70.1, 4 bit 80.7 -> 78.1, 8 bit 83.9 -> 80.1; half 8 bit
-// with 4 workgroups 66.4 -> 63.7; quantize float 2 bit with 10 one-wave workgroups 71.5 -> 69.5, 4 bit with
-// 16: 75.6 -> 72.8.  The other kernels (all half quantize, float quantize at 1 and 8 bit) and small tensors
-// gain nothing or lose, and keep full occupancy.
+// Interleaved A/B in both orders on a 411 MB float tensor (us, full occupancy -> capped): dequantize with
+// 3 workgroups of 4 waves per CU 1 bit 77.3 -> 64.5, 2 bit 76.3 -> 69.0, 4 bit 80.0 -> 77.8, 8 bit 83.2 -> 79.3;
+// half 8 bit with 4 workgroups 65.8 -> 62.7; quantize float 4 bit with 16 one-wave workgroups 76.1 -> 71.1.
+// The other kernels (all half quantize, float quantize at 1, 2 and 8 bit) and small tensors gain nothing or
+// lose, and keep full occupancy.
 constexpr int64_t kCapFromGroups = 1 << 16;  // 16.8 M elements
 inline unsigned dequantize_lds_cap(size_t elem_size, int bits, int64_t N) {
   if (N < kCapFromGroups) return 0u;
@@ -1368,7 +1368,7 @@ inline unsigned dequantize_lds_cap(size_t elem_size, int bits, int64_t N) {
 }
 inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
   if (elem_size != 4 || N < kCapFromGroups) return 0u;
-  return bits == 2 ? 16000u : bits == 4 ? 10000u : 0u;
+  return bits == 4 ? 10000u : 0u;
 }
 
 template <typename T, int BITS, bool GIVEN>
