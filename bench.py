@@ -30,8 +30,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # a copy kernel of known size (profiles/config2_fp32_4bit_quantize_dequantize.txt: the copy kernel reads
 # FETCH_SIZE x 1.99988 and WRITE_SIZE x 1.00000 KiB); None for workloads without a counter run
 TRAFFIC_BYTES = {
-    ("config2", "quantize"): 466.8e6,    # 411.1 MB read + 55.7 MB written; algorithmic 465.6 MB
-    ("config2", "dequantize"): 465.8e6,  # 54.7 MB read + 411.1 MB written; algorithmic 465.6 MB
+    ("config2", "quantize"): 466.5e6,    # 411.1 MB read + 55.4 MB written; algorithmic 465.6 MB
+    ("config2", "dequantize"): 465.7e6,  # 54.7 MB read + 411.1 MB written; algorithmic 465.6 MB
 }
 
 # a workload whose buffers are smaller than this is timed over several buffer sets in rotation
