@@ -187,12 +187,15 @@ def test_calc_precision_device_reports_unreachable_budget():
     assert status.item() == -5 and b.cpu().tolist() == [1] * L
 
 
-@pytest.mark.parametrize("stream", ["deterministic", "fast", "reference"])
-def test_batched_equals_tensor_by_tensor(stream):
+@pytest.mark.parametrize("stream,mix", [("deterministic", "both"), ("fast", "both"), ("reference", "both"),
+                                        ("fast", "float"), ("fast", "half")])
+def test_batched_equals_tensor_by_tensor(stream, mix):
     rng = np.random.default_rng(3)
     L = 24
     shapes = _swin_like(rng, L) + [(100, 77), (3, 5)]
-    dtypes = [torch.float16 if i % 3 else torch.float32 for i in range(len(shapes))]
+    # element types of the table: mixed, or one type only (then only that type's kernels are launched)
+    dtypes = [{"float": torch.float32, "half": torch.float16}.get(mix, torch.float16 if i % 3 else torch.float32)
+              for i in range(len(shapes))]
     L = len(shapes)
     g = torch.Generator().manual_seed(0)
     tensors = [torch.randn(s, generator=g).to(d).cuda() for s, d in zip(shapes, dtypes)]
@@ -203,6 +206,7 @@ def test_batched_equals_tensor_by_tensor(stream):
                                                     torch.from_numpy(C).cuda(), torch.from_numpy(w).cuda(), target)
     seeds = [i + 5 for i in range(L)]
     bq = BatchedQuantizer([t.numel() for t in tensors], dtypes, "cuda")
+    assert bq.dtype_mask == {"both": 3, "float": 1, "half": 2}[mix]
     q = bq.quantize(tensors, bits, seeds, arena_bytes=bq.arena_bytes_for_budget(target), rng_stream=stream)
     ok, need = q.ok()
     assert ok and need <= q.packed.numel()
