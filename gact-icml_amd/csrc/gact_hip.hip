@@ -1032,11 +1032,12 @@ __host__ __device__ inline float prec_key(float C, int b, int64_t w) {
 __host__ __device__ inline bool prec_valid_bits(int b) { return b == 1 || b == 2 || b == 4 || b == 8 || b == 32; }
 
 #define PREC_MAX_L 4096      /* tensors the device kernel handles (LDS tables) */
-#define PREC_SORT_MAX_L 1024 /* tensors the sorting path handles (4 candidate steps each) */
+#define PREC_SORT_MAX_L 4096 /* tensors the sorting path handles (4 candidate steps each, 8 bytes per candidate) */
+#define PREC_THREADS 1024    /* largest workgroup the kernel is launched with */
 
-// The sequential restatement of the heap loop by one wave: each step is a 64-lane argmax.  Used when the
-// table is too long for the sorting path or a tensor's step keys do not decrease (never the case for the
-// non-negative sensitivities the callers produce).
+// The sequential restatement of the heap loop by one wave: each step is a 64-lane argmax.  Used when a
+// tensor's step keys do not decrease (never the case for the finite positive sensitivities the callers
+// produce).
 __device__ void calc_precision_sequential(int32_t* __restrict__ b_s, float* __restrict__ key_s,
                                           const float* __restrict__ C, const int64_t* __restrict__ w, int L,
                                           double b_sum, double target, int* rc_out) {
@@ -1086,28 +1087,30 @@ __device__ __forceinline__ uint32_t sortable_key(float k) {
 // The greedy pops candidates (tensor i, step s) in descending (key, i) order.  A tensor's steps have
 // strictly decreasing keys, so that order is the descending sort of ALL candidate steps by
 // (key, index, earlier step first); the loop `while (b_sum > target) pop` then takes a prefix of it.
-// 256 threads: build up to 4 candidates per tensor, bitonic-sort them in LDS, prefix-sum the savings
-// (integers, exact in double), apply the prefix.  Falls back to the sequential loop when that order
-// argument does not hold.
-__global__ void __launch_bounds__(256)
+// One workgroup of 256 or 1024 threads: build up to 4 candidates per tensor, bitonic-sort them in LDS,
+// prefix-sum the savings (integers, exact in double), apply the prefix.  Falls back to the sequential
+// loop when that order argument does not hold.
+__global__ void __launch_bounds__(PREC_THREADS)
 calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, const int64_t* __restrict__ w,
                       int L, double target, int32_t* __restrict__ status) {
-  __shared__ uint64_t cand[4 * PREC_SORT_MAX_L];  // 32 KB; the sequential path reuses it for its float keys
+  // dynamic LDS: one 8-byte slot per candidate, 4 per tensor rounded up to a power of two (128 KB for 4096
+  // tensors); the sequential path reuses it for its float keys
+  extern __shared__ uint64_t cand[];
   __shared__ int32_t b_s[PREC_MAX_L];
-  __shared__ double part_s[256];
+  __shared__ double part_s[PREC_THREADS];
   __shared__ int flag_s;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, NT = blockDim.x;
   const bool sortable = L <= PREC_SORT_MAX_L;
   int M = 4;
   while (M < 4 * L) M <<= 1;
   if (tid == 0) flag_s = 0;
   if (sortable)
-    for (int t = tid; t < M; t += 256) cand[t] = 0;  // 0 sorts after every real candidate
+    for (int t = tid; t < M; t += NT) cand[t] = 0;  // 0 sorts after every real candidate
   __syncthreads();
 
   double part = 0.0;
   bool bad_order = false, bad_width = false;
-  for (int idx = tid; idx < L; idx += 256) {
+  for (int idx = tid; idx < L; idx += NT) {
     const int bi = b[idx];
     b_s[idx] = bi;
     if (!prec_valid_bits(bi)) {
@@ -1141,7 +1144,7 @@ calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, cons
     return;
   }
   // every term is an integer; the sum is exact (and order-free) below 2^53
-  for (int off = 128; off >= 1; off >>= 1) {
+  for (int off = NT >> 1; off >= 1; off >>= 1) {
     if (tid < off) part_s[tid] += part_s[tid + off];
     __syncthreads();
   }
@@ -1156,7 +1159,7 @@ calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, cons
     // bitonic sort, descending
     for (int k = 2; k <= M; k <<= 1) {
       for (int j = k >> 1; j > 0; j >>= 1) {
-        for (int t = tid; t < M; t += 256) {
+        for (int t = tid; t < M; t += NT) {
           const int o = t ^ j;
           if (o > t) {
             const uint64_t x = cand[t], y = cand[o];
@@ -1168,7 +1171,7 @@ calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, cons
       }
     }
     // savings of the sorted candidates, chunked over the threads
-    const int per = M / 256 > 0 ? M / 256 : 1;
+    const int per = M / NT > 0 ? M / NT : 1;
     const int lo = tid * per, hi = lo + per < M ? lo + per : M;
     double mine = 0.0;
     for (int t = lo; t < hi && t < M; t++) {
@@ -1181,9 +1184,9 @@ calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, cons
     }
     part_s[tid] = (lo < M) ? mine : 0.0;
     __syncthreads();
-    if (tid == 0) {  // exclusive prefix over 256 partial sums
+    if (tid == 0) {  // exclusive prefix over the partial sums
       double run = 0.0;
-      for (int t = 0; t < 256; t++) { const double v = part_s[t]; part_s[t] = run; run += v; }
+      for (int t = 0; t < NT; t++) { const double v = part_s[t]; part_s[t] = run; run += v; }
       if (b_sum0 - run > target) flag_s = 2;  // every step taken and still over budget
     }
     __syncthreads();
@@ -1202,7 +1205,7 @@ calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, cons
     if (flag_s == 2) rc = GACT_EBUDGET;
   }
   __syncthreads();
-  for (int idx = tid; idx < L; idx += 256) b[idx] = b_s[idx];
+  for (int idx = tid; idx < L; idx += NT) b[idx] = b_s[idx];
   if (status && tid == 0) *status = rc;
 }
 
@@ -1635,7 +1638,15 @@ int gact_calc_precision_device(int32_t* b, const float* C, const int64_t* w, int
   if (L > PREC_MAX_L) return GACT_ESHAPE;
   if (L == 0) return GACT_OK;
   if (!b || !C || !w) return GACT_EINVAL;
-  hipLaunchKernelGGL(calc_precision_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, b, C, w, (int)L, target, status);
+  int64_t M = 4;
+  while (M < 4 * L) M <<= 1;
+  const size_t lds = (size_t)M * sizeof(uint64_t);
+  if (lds > 48 * 1024 &&
+      hipFuncSetAttribute((const void*)calc_precision_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+          hipSuccess)
+    return GACT_ELAUNCH;
+  hipLaunchKernelGGL(calc_precision_kernel, dim3(1), dim3(L <= 256 ? 256 : PREC_THREADS), lds, (hipStream_t)stream, b, C, w,
+                     (int)L, target, status);
   return launch_status();
 }
 

@@ -155,9 +155,15 @@ def test_calc_precision_device_adversarial_orders():
     cases.append((np.zeros(50, np.float32), np.full(50, 1024, np.int64), 8, 2.0))
     cases.append((np.array([0.0, 1.0, 0.0, 2.0, 0.0], np.float32), np.full(5, 512, np.int64), 32, 2.0))
     cases.append((np.array([np.inf, 1.0, np.inf, 2.0], np.float32), np.full(4, 512, np.int64), 8, 2.0))
-    big = 1500                                       # beyond the sorting path: the sequential path
-    cases.append((np.exp(rng.normal(0, 2, big)).astype(np.float32), (rng.integers(1, 50, big) * 256).astype(np.int64), 8, 2.0))
-    cases.append((np.exp(rng.normal(0, 2, 1024)).astype(np.float32), (rng.integers(1, 50, 1024) * 256).astype(np.int64), 32, 3.0))
+    # long tables: the sorting path up to its limit of 4096 tensors (1024 threads, 128 KB of LDS), and the
+    # sequential path at a length only it is asked to handle (an infinite sensitivity leaves the sorting path)
+    for big, init, avg in ((1500, 8, 2.0), (1024, 32, 3.0), (4096, 8, 1.5), (3000, 32, 2.5)):
+        cases.append((np.exp(rng.normal(0, 2, big)).astype(np.float32), (rng.integers(1, 50, big) * 256).astype(np.int64), init, avg))
+    C_inf = np.exp(rng.normal(0, 2, 1500)).astype(np.float32)
+    C_inf[700] = np.inf
+    cases.append((C_inf, (rng.integers(1, 50, 1500) * 256).astype(np.int64), 8, 2.0))
+    ties = np.full(2500, 1.0, np.float32)            # every key equal: the order is decided by the index alone
+    cases.append((ties, np.full(2500, 4096, np.int64), 8, 3.0))
     for C, w, init, avg in cases:
         L = C.size
         target = avg * float(w.sum())
