@@ -25,6 +25,7 @@
 #include <stdint.h>
 
 #include <queue>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
@@ -856,27 +857,55 @@ minimax256_kernel(const T* __restrict__ x, int64_t N, T* __restrict__ mn, T* __r
 // General shapes (any D for minimax; any G, D for pack / unpack).  These keep the operator surface
 // complete; the path the library is built for is G = 1, D = 256 above.
 // ------------------------------------------------------------------------------------------------
-template <typename T>
+// Row min/max for any D.  2^lpr_log2 lanes share a row (8..64: as many as the row has 16-byte pieces, so
+// short rows put several rows in a wave) and a lane group takes R consecutive rows, all of whose loads are
+// issued before the first reduction.  VEC = false (a base address that is not 16-byte aligned) reads
+// element by element.
+template <typename T, bool VEC, int R>
 __global__ void __launch_bounds__(256)
-minimax_any_kernel(const T* __restrict__ x, int64_t N, int64_t D, T* __restrict__ mn, T* __restrict__ mx) {
-  // one wave per row
-  const int64_t n = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (n >= N) return;
-  const int lane = threadIdx.x & 63;
-  float lo = Elem<T>::init_lo(), hi = Elem<T>::init_hi();
-  for (int64_t d = lane; d < D; d += 64) {
-    float f = (float)x[n * D + d];
-    lo = __builtin_fminf(lo, f);
-    hi = __builtin_fmaxf(hi, f);
+minimax_any_kernel(const T* __restrict__ x, int64_t N, int64_t D, int lpr_log2, T* __restrict__ mn,
+                   T* __restrict__ mx) {
+  constexpr int W = VEC ? 16 / (int)sizeof(T) : 1;
+  typedef T vecw __attribute__((ext_vector_type(VEC ? W : 2)));
+  typedef typename std::conditional<VEC, vecw, T>::type vec;
+  const int lpr = 1 << lpr_log2;
+  const int64_t group = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> lpr_log2;
+  const int sub = threadIdx.x & (lpr - 1);
+  const int64_t V = D / W;
+  float lo[R], hi[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    lo[r] = Elem<T>::init_lo();
+    hi[r] = Elem<T>::init_hi();
+    const int64_t n = group * R + r;
+    if (n < N) {
+      const vec* row = reinterpret_cast<const vec*>(x + n * D);
+#pragma unroll 4
+      for (int64_t v = sub; v < V; v += lpr) {
+        const vec q = stream_load(row + v);
+#pragma unroll
+        for (int e = 0; e < W; e++) {
+          float f;
+          if constexpr (VEC) f = (float)q[e]; else f = (float)q;
+          lo[r] = __builtin_fminf(lo[r], f);
+          hi[r] = __builtin_fmaxf(hi[r], f);
+        }
+      }
+    }
   }
 #pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    lo = __builtin_fminf(lo, __shfl_xor(lo, off, 64));
-    hi = __builtin_fmaxf(hi, __shfl_xor(hi, off, 64));
-  }
-  if (lane == 0) {
-    mn[n] = Elem<T>::from_float(lo);
-    mx[n] = Elem<T>::from_float(hi);
+  for (int r = 0; r < R; r++) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1)
+      if (off < lpr) {  // uniform over the launch
+        lo[r] = __builtin_fminf(lo[r], __shfl_xor(lo[r], off, 64));
+        hi[r] = __builtin_fmaxf(hi[r], __shfl_xor(hi[r], off, 64));
+      }
+    const int64_t n = group * R + r;
+    if (sub == 0 && n < N) {
+      mn[n] = Elem<T>::from_float(lo[r]);
+      mx[n] = Elem<T>::from_float(hi[r]);
+    }
   }
 }
 
@@ -954,27 +983,46 @@ unpack_any_kernel(const uint8_t* __restrict__ packed, int bits, const T* __restr
 // (low and high half of each ballot).  A partial last block is packed sequentially (element e -> word
 // e/32, bit e%32), which is the plain ballot of one byte per lane and fits the ceil(n/32)-word output.
 // ------------------------------------------------------------------------------------------------
+// A wave takes MASK_PAIRS consecutive pairs of blocks (4 KB of mask bytes) and issues all its loads first.
+#define MASK_PAIRS 4
 __global__ void __launch_bounds__(256)
 mask_pack_kernel(const uint8_t* __restrict__ data, int64_t n, int32_t* __restrict__ mask) {
   const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int64_t full_blocks = n / 512;
-  const int64_t blk0 = wave * 2;  // this wave packs blocks blk0 and blk0 + 1
-  if (blk0 < full_blocks) {
-    const bool have = (blk0 + (lane >> 5)) < full_blocks;
-    u32x4 q = {0u, 0u, 0u, 0u};
-    if (have) q = *reinterpret_cast<const u32x4*>(data + (blk0 * 32 + lane) * 16);
-    uint32_t mine = 0;
+  const int64_t pairs = (full_blocks + 1) / 2;
+  const int64_t pair0 = wave * MASK_PAIRS;
+  if (pair0 < pairs) {
+    u32x4 q[MASK_PAIRS];
 #pragma unroll
-    for (int w = 0; w < 16; w++) {
-      const uint32_t word = w < 4 ? q.x : w < 8 ? q.y : w < 12 ? q.z : q.w;
-      const uint64_t b = __ballot(((word >> (8 * (w & 3))) & 0xffu) != 0u);
-      if ((lane & 15) == w) mine = (lane & 16) ? (uint32_t)(b >> 32) : (uint32_t)b;
+    for (int j = 0; j < MASK_PAIRS; j++) {
+      const int64_t blk = (pair0 + j) * 2 + (lane >> 5);  // lanes 0..31 hold the pair's first block
+      q[j] = u32x4{0u, 0u, 0u, 0u};
+      if (blk < full_blocks) q[j] = stream_load(reinterpret_cast<const u32x4*>(data + (blk * 32 + (lane & 31)) * 16));
     }
-    if (lane < 32 && (blk0 + (lane >> 4)) < full_blocks) mask[blk0 * 16 + lane] = (int32_t)mine;
+    // word w of a block is the ballot of "byte w is nonzero" over the block's 32 lanes.  The 32 words of
+    // pair j are collected in lanes 32 * (j & 1) ..: one store then writes two pairs.
+    uint32_t mine[MASK_PAIRS / 2];
+#pragma unroll
+    for (int j = 0; j < MASK_PAIRS; j++) {
+      uint32_t sel = 0;
+#pragma unroll
+      for (int w = 0; w < 16; w++) {
+        const uint32_t word = w < 4 ? q[j].x : w < 8 ? q[j].y : w < 12 ? q[j].z : q[j].w;
+        const uint64_t b = __ballot(((word >> (8 * (w & 3))) & 0xffu) != 0u);
+        if ((lane & 15) == w) sel = (lane & 16) ? (uint32_t)(b >> 32) : (uint32_t)b;
+      }
+      if ((j & 1) == 0) mine[j >> 1] = sel;
+      else if (lane >= 32) mine[j >> 1] = sel;
+    }
+#pragma unroll
+    for (int jj = 0; jj < MASK_PAIRS / 2; jj++) {
+      const int64_t word = (pair0 + 2 * jj) * 32 + lane;  // 16 words per block
+      if ((word >> 4) < full_blocks) stream_store(mine[jj], reinterpret_cast<uint32_t*>(mask) + word);
+    }
   }
-  // the partial block goes to the wave after the last full pair
-  if (wave == (full_blocks + 1) / 2) {
+  // the partial block goes to the wave after the last one that packs full blocks
+  if (wave == (pairs + MASK_PAIRS - 1) / MASK_PAIRS) {
     const int64_t base = full_blocks * 512;
     const int64_t words = (n + 31) / 32;
     for (int64_t e0 = base; e0 < n; e0 += 64) {
@@ -987,26 +1035,48 @@ mask_pack_kernel(const uint8_t* __restrict__ data, int64_t n, int32_t* __restric
   }
 }
 
+// A thread writes 16 elements (bit k of the 16 words of its block); a wave covers a pair of blocks per
+// step and takes MASK_PAIRS steps, all loads first.
 __global__ void __launch_bounds__(256)
 mask_unpack_kernel(const int32_t* __restrict__ mask, int64_t n, uint8_t* __restrict__ out) {
-  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // 16 elements per thread
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
   const int64_t full_blocks = n / 512;
-  const int64_t blk = t >> 5;
-  const int k = (int)(t & 31);
-  if (blk < full_blocks) {
-    uint32_t q[4] = {0u, 0u, 0u, 0u};
+  const int k = lane & 31;
+  const bool vec = (reinterpret_cast<uintptr_t>(mask) & 15u) == 0;
+  u32x4 m[MASK_PAIRS][4];
 #pragma unroll
-    for (int w = 0; w < 16; w++) {
-      const uint32_t bit = ((uint32_t)mask[blk * 16 + w] >> k) & 1u;
-      q[w >> 2] |= bit << (8 * (w & 3));
+  for (int j = 0; j < MASK_PAIRS; j++) {
+    const int64_t blk = (wave * MASK_PAIRS + j) * 2 + (lane >> 5);
+    if (blk < full_blocks) {
+      if (vec) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) m[j][c] = reinterpret_cast<const u32x4*>(mask + blk * 16)[c];
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          const uint32_t* p = reinterpret_cast<const uint32_t*>(mask) + blk * 16 + c * 4;
+          m[j][c] = u32x4{p[0], p[1], p[2], p[3]};
+        }
+      }
     }
-    u32x4 v = {q[0], q[1], q[2], q[3]};
-    *reinterpret_cast<u32x4*>(out + t * 16) = v;
-  } else if (blk == full_blocks) {
-    const int64_t base = full_blocks * 512;
-    for (int64_t e = base + k * 16; e < base + k * 16 + 16 && e < n; e++) {
-      const int64_t r = e - base;
-      out[e] = (uint8_t)(((uint32_t)mask[full_blocks * 16 + r / 32] >> (r % 32)) & 1u);
+  }
+#pragma unroll
+  for (int j = 0; j < MASK_PAIRS; j++) {
+    const int64_t blk = (wave * MASK_PAIRS + j) * 2 + (lane >> 5);
+    if (blk < full_blocks) {
+      uint32_t q[4];
+#pragma unroll
+      for (int c = 0; c < 4; c++)
+        q[c] = ((m[j][c].x >> k) & 1u) | (((m[j][c].y >> k) & 1u) << 8) | (((m[j][c].z >> k) & 1u) << 16) |
+               (((m[j][c].w >> k) & 1u) << 24);
+      stream_store(u32x4{q[0], q[1], q[2], q[3]}, reinterpret_cast<u32x4*>(out + (blk * 32 + k) * 16));
+    } else if (blk == full_blocks) {
+      const int64_t base = full_blocks * 512;
+      for (int64_t e = base + k * 16; e < base + k * 16 + 16 && e < n; e++) {
+        const int64_t r = e - base;
+        out[e] = (uint8_t)(((uint32_t)mask[full_blocks * 16 + r / 32] >> (r % 32)) & 1u);
+      }
     }
   }
 }
@@ -1435,6 +1505,25 @@ int dispatch_dequantize(int bits, const uint8_t* packed, const T* scale, const T
 }
 
 template <typename T>
+void launch_minimax_any(const T* x, int64_t N, int64_t D, T* mn, T* mx, hipStream_t stream) {
+  const bool vec = aligned16(x);  // D % 32 == 0 keeps every row 16-byte aligned once the base is
+  const int64_t pieces = vec ? D / (16 / (int64_t)sizeof(T)) : D;
+  int lpr_log2 = 3;
+  while (lpr_log2 < 6 && (2LL << lpr_log2) <= pieces) lpr_log2++;
+  const bool several = pieces <= (64LL << 1);  // short rows: 4 rows per lane group
+  const int64_t groups = several ? (N + 3) / 4 : N;
+  const dim3 grid((unsigned)(((groups << lpr_log2) + 255) / 256)), block(256);
+  if (vec && several)
+    hipLaunchKernelGGL((minimax_any_kernel<T, true, 4>), grid, block, 0, stream, x, N, D, lpr_log2, mn, mx);
+  else if (vec)
+    hipLaunchKernelGGL((minimax_any_kernel<T, true, 1>), grid, block, 0, stream, x, N, D, lpr_log2, mn, mx);
+  else if (several)
+    hipLaunchKernelGGL((minimax_any_kernel<T, false, 4>), grid, block, 0, stream, x, N, D, lpr_log2, mn, mx);
+  else
+    hipLaunchKernelGGL((minimax_any_kernel<T, false, 1>), grid, block, 0, stream, x, N, D, lpr_log2, mn, mx);
+}
+
+template <typename T>
 int pack_any(const T* data, const T* mn, const T* scale, int bits, int64_t N, int64_t G, int64_t D, int noise_mode,
              uint64_t seed, const float* noise, uint8_t* packed, hipStream_t stream) {
   const int64_t total = gact_packed_bytes(bits, N, G, D);
@@ -1497,11 +1586,10 @@ int gact_minimax(const void* data, int dtype, int64_t N, int64_t D, void* mn, vo
     else
       hipLaunchKernelGGL((minimax256_kernel<f16>), grid, block, 0, s, (const f16*)data, N, (f16*)mn, (f16*)mx);
   } else {
-    const dim3 grid((unsigned)((N + 3) / 4)), block(256);
     if (dtype == GACT_F32)
-      hipLaunchKernelGGL((minimax_any_kernel<float>), grid, block, 0, s, (const float*)data, N, D, (float*)mn, (float*)mx);
+      launch_minimax_any<float>((const float*)data, N, D, (float*)mn, (float*)mx, s);
     else
-      hipLaunchKernelGGL((minimax_any_kernel<f16>), grid, block, 0, s, (const f16*)data, N, D, (f16*)mn, (f16*)mx);
+      launch_minimax_any<f16>((const f16*)data, N, D, (f16*)mn, (f16*)mx, s);
   }
   return launch_status();
 }
@@ -1591,8 +1679,8 @@ int gact_mask_pack(const uint8_t* data, int64_t n, int32_t* mask, void* stream) 
   if (n == 0) return GACT_OK;
   if (!data || !mask) return GACT_EINVAL;
   if (!aligned16(data)) return GACT_EALIGN;
-  const int64_t full_blocks = n / 512;
-  const int64_t waves = (full_blocks + 1) / 2 + 1;  // pairs of full blocks, plus the one that takes the partial block
+  const int64_t pairs = (n / 512 + 1) / 2;  // pairs of full blocks
+  const int64_t waves = (pairs + MASK_PAIRS - 1) / MASK_PAIRS + 1;  // plus the wave that takes the partial block
   hipLaunchKernelGGL(mask_pack_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, (hipStream_t)stream, data, n, mask);
   return launch_status();
 }
@@ -1602,8 +1690,9 @@ int gact_mask_unpack(const int32_t* mask, int64_t n, uint8_t* out, void* stream)
   if (n == 0) return GACT_OK;
   if (!mask || !out) return GACT_EINVAL;
   if (!aligned16(out)) return GACT_EALIGN;
-  const int64_t threads = (n / 512 + 1) * 32;
-  hipLaunchKernelGGL(mask_unpack_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, (hipStream_t)stream, mask, n, out);
+  const int64_t pairs = (n / 512 + 2) / 2;  // pairs of blocks, the partial block included
+  const int64_t waves = (pairs + MASK_PAIRS - 1) / MASK_PAIRS;
+  hipLaunchKernelGGL(mask_unpack_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, (hipStream_t)stream, mask, n, out);
   return launch_status();
 }
 

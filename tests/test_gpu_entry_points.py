@@ -35,6 +35,19 @@ def test_minimax(dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f16"])
+@pytest.mark.parametrize("shape", [(41, 64), (7, 256), (6, 1024), (11, 160)])
+def test_minimax_on_a_base_address_that_is_not_16_byte_aligned(dtype, shape):
+    # a contiguous view one element into a buffer: the element-by-element variant of the kernel
+    N, D = shape
+    g = torch.Generator().manual_seed(2)
+    buf = torch.randn(N * D + 1, generator=g).to(dtype).cuda()
+    x = buf[1:].view(N, D)
+    assert x.is_contiguous() and x.data_ptr() % 16 != 0
+    mn, mx = ext_minimax.minimax(x)
+    assert torch.equal(mn, x.min(dim=1).values) and torch.equal(mx, x.max(dim=1).values)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f16"])
 @pytest.mark.parametrize("bits", [1, 2, 4, 8])
 @pytest.mark.parametrize("ngd", [(203, 1, 256), (21, 3, 64), (10, 2, 256), (9, 1, 128)])
 @pytest.mark.parametrize("stream", ["deterministic", "reference", "fast"])
@@ -109,6 +122,20 @@ def test_dropout_mask(n):
     np.testing.assert_array_equal(q[0].cpu().numpy(), oracle.mask_pack(data.numpy()))
     out = ops.op_dequantize_mask(q)
     assert out.dtype == torch.uint8 and torch.equal(out.cpu(), data)
+
+
+def test_dropout_mask_every_count_of_blocks_a_wave_can_end_on():
+    # a wave takes 8 blocks of 512 elements: every residue of the block count, with and without a partial block
+    g = torch.Generator().manual_seed(5)
+    for blocks in range(0, 18):
+        for rest in (0, 1, 33, 511):
+            n = 512 * blocks + rest
+            if n == 0:
+                continue
+            data = (torch.rand(n, generator=g) < 0.5).to(torch.uint8)
+            q = ops.op_quantize_mask(data.cuda())
+            np.testing.assert_array_equal(q[0].cpu().numpy(), oracle.mask_pack(data.numpy()), err_msg="n=%d" % n)
+            assert torch.equal(ops.op_dequantize_mask(q).cpu(), data), n
 
 
 def test_dropout_mask_one_hot_identity():
