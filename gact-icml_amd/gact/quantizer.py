@@ -8,7 +8,7 @@ import torch
 
 from .conf import config
 from .ops import op_dequantize, op_dequantize_mask, op_quantize, op_quantize_mask
-from .utils import uniform_sample
+from .utils import sampled_key_with_sum
 
 _COMPRESSIBLE = (torch.float32, torch.float16)
 _RANKS = (2, 3, 4)
@@ -86,7 +86,7 @@ class Quantizer:
         if not config.check_dup:
             return tid
         # the same tensor saved by two operators: address + strided sample + sum
-        return tuple(uniform_sample(t, min(KEY_SAMPLES, t.numel()), add_dataptr=True) + [t.sum().item()])
+        return tuple(sampled_key_with_sum(t, KEY_SAMPLES))
 
     def iterate(self):
         self.ptr_qtensor_map, self.layer_key_map = {}, {}

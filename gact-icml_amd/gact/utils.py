@@ -26,6 +26,18 @@ def uniform_sample(input, sample_cnt, add_dataptr=True):
     return _key_prefix(input, add_dataptr) + input.ravel()[positions].tolist()
 
 
+def sampled_key_with_sum(input, sample_cnt):
+    """uniform_sample(input, sample_cnt) + [input.sum().item()] with one device-to-host copy instead of two:
+    the samples and the sum travel together as float64, which holds float16 and float32 values exactly."""
+    n = input.numel()
+    take = min(n, sample_cnt)
+    total = input.sum().to(torch.float64).reshape(1)
+    if take == 0:
+        return _key_prefix(input, True) + total.tolist()
+    positions = torch.arange(take, device=input.device) * (n // take)
+    return _key_prefix(input, True) + torch.cat([input.ravel()[positions].to(torch.float64), total]).tolist()
+
+
 def uniform_sample_ref(input, sample_cnt, add_dataptr=True):
     """The same key read value by value; what uniform_sample is tested against."""
     stride = max(input.numel() // sample_cnt, 1)

@@ -4,8 +4,8 @@ import json
 
 import torch
 
-from gact.utils import (GlobalExpRecorder, compute_tensor_bytes, empty_cache, random_sample, uniform_sample,
-                        uniform_sample_ref)
+from gact.utils import (GlobalExpRecorder, compute_tensor_bytes, empty_cache, random_sample, sampled_key_with_sum,
+                        uniform_sample, uniform_sample_ref)
 
 
 def sample_by_loop(t, cnt, add_dataptr=True):
@@ -24,6 +24,14 @@ def test_uniform_sample_matches_a_plain_loop():
         assert uniform_sample(t, cnt, add_dataptr=False) == sample_by_loop(t, cnt, add_dataptr=False)
         assert uniform_sample(t, cnt) == uniform_sample_ref(t, cnt)
     assert uniform_sample(torch.empty(0), 10, add_dataptr=False) == []
+
+
+def test_key_with_sum_equals_the_two_step_key():
+    # the duplicate-detection key of gact/gact/quantizer.py:85-93: address, strided sample, sum
+    for dtype in (torch.float32, torch.float16):
+        for n in (1, 7, 100, 1000, 4097):
+            t = torch.randn(n).to(dtype)
+            assert sampled_key_with_sum(t, 100) == uniform_sample(t, min(100, n)) + [t.sum().item()]
 
 
 def test_random_sample_is_reproducible_and_leaves_the_global_stream_alone():
