@@ -622,35 +622,22 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
   }
 
   if constexpr (BITS <= 4) {
-    // A group has only 2^BITS distinct outputs T(c)/scale + min.  The 16 lanes of a row tabulate them - one
-    // entry per lane, 16/2^BITS groups per pass, with the real division and the real sum - and every element
-    // then fetches its value from the lane that holds it (ds_bpermute: the LDS crossbar, no LDS memory).
-    // 2 vector instructions per element instead of 6, and the division runs once per table entry.
-    constexpr int ENT = 1 << BITS, GPP = 16 / ENT, PASSES = G / GPP;
-    const float cf = (float)(rl & (ENT - 1));
+    // A group has only 2^BITS distinct outputs T(c)/scale + min: 8 * 2^BITS values for the unit.  Its lanes
+    // tabulate them - entry e = group * 2^BITS + code in lane e % LPU, pass e / LPU, each with the real
+    // division and the real sum - and every element then fetches its value from the lane that holds it
+    // (ds_bpermute: the LDS crossbar, no LDS memory).  2 vector instructions per element instead of 6, and
+    // one or two divisions per lane (four for half at 4 bit) instead of one per element.
+    constexpr int LPU = GROUP / W;
+    constexpr int ENT = 1 << BITS, TOT = G * ENT, PASSES = (TOT + LPU - 1) / LPU;
     uint32_t tab[PASSES];
-    constexpr int PER16 = 16 / (int)sizeof(T);
-    if (GPP == 1 && G % PER16 == 0 && g0 + G <= N &&
-        ((reinterpret_cast<uintptr_t>(scale + g0) | reinterpret_cast<uintptr_t>(mn + g0)) & 15u) == 0) {
-      // one group per pass: every lane needs all 8 scales and minima, two 16-byte loads each instead of 16 small ones
-      typedef T vec16 __attribute__((ext_vector_type(PER16)));
-      vec16 sv[G / PER16], mv[G / PER16];
 #pragma unroll
-      for (int c = 0; c < G / PER16; c++) {
-        sv[c] = *reinterpret_cast<const vec16*>(scale + g0 + c * PER16);
-        mv[c] = *reinterpret_cast<const vec16*>(mn + g0 + c * PER16);
-      }
-#pragma unroll
-      for (int p = 0; p < PASSES; p++) tab[p] = Elem<T>::table_entry(cf, sv[p / PER16][p % PER16], mv[p / PER16][p % PER16]);
-    } else {
-#pragma unroll
-      for (int p = 0; p < PASSES; p++) {
-        const int64_t g = g0 + p * GPP + rl / ENT;
-        const bool live = g < N;
-        tab[p] = Elem<T>::table_entry(cf, live ? scale[g] : (T)1, live ? mn[g] : (T)0);
-      }
+    for (int p = 0; p < PASSES; p++) {
+      const int e = p * LPU + l;
+      const int64_t g = g0 + e / ENT;
+      const bool live = e < TOT && g < N;
+      tab[p] = Elem<T>::table_entry((float)(e & (ENT - 1)), live ? scale[g] : (T)1, live ? mn[g] : (T)0);
     }
-    const uint32_t rowbase = threadIdx.x & 48u;
+    const uint32_t unitbase = (threadIdx.x & 63u) & ~(uint32_t)(LPU - 1);  // first lane of the unit within its wave
 #pragma unroll
     for (int it = 0; it < SGS; it++) {
 #pragma unroll
@@ -658,12 +645,12 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
         const int64_t n = (sg0 + it) * WPT + ni;
         if (n < N) {
           const int g = it * WPT + ni;
-          const uint32_t base4 = (rowbase + (uint32_t)(g % GPP) * ENT) << 2;
+          const uint32_t base4 = (unitbase + (uint32_t)((g * ENT) % LPU)) << 2;
           T v[W];
 #pragma unroll
           for (int e = 0; e < W; e++) {
             const uint32_t c = __builtin_amdgcn_ubfe(w[it][e >> 2], 8 * (e & 3) + ni * BITS, BITS);
-            v[e] = Elem<T>::from_bits((uint32_t)__builtin_amdgcn_ds_bpermute((int)((c << 2) + base4), (int)tab[g / GPP]));
+            v[e] = Elem<T>::from_bits((uint32_t)__builtin_amdgcn_ds_bpermute((int)((c << 2) + base4), (int)tab[(g * ENT) / LPU]));
           }
           const int64_t at = n * GROUP + W * l;
           if (n * GROUP + GROUP <= numel) {
