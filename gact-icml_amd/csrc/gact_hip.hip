@@ -963,6 +963,88 @@ unpack_any_kernel(const uint8_t* __restrict__ packed, int bits, const T* __restr
   }
 }
 
+// G = 1 and D a multiple of 8 (every group size config.group_size can take): a thread owns 8 consecutive
+// columns of one super-group - 8 output bytes, 8 elements of each of its 8/bits groups with 16-byte loads -
+// and no thread divides 64-bit indices.  Same arithmetic and the same noise streams as pack_any_kernel.
+template <typename T, int NOISE>
+__global__ void __launch_bounds__(256)
+pack_rows8_kernel(const T* __restrict__ data, const T* __restrict__ mn, const T* __restrict__ scale, int bits,
+                  int64_t N, uint32_t tpr /* threads per super-group = D / 8 */, uint32_t total_threads, uint64_t seed,
+                  const float* __restrict__ noise, uint8_t* __restrict__ packed) {
+  const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= total_threads) return;
+  const int wpt = 8 / bits;
+  const uint32_t no = t / tpr, c8 = t - no * tpr;
+  const int64_t D = (int64_t)tpr * 8;
+  const int64_t j0 = (int64_t)no * D + (int64_t)c8 * 8;  // first output byte
+  const uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+  typedef T vec8 __attribute__((ext_vector_type(8)));
+  uint32_t bytes[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+  uint32_t r[8][4];
+  for (int ni = 0; ni < wpt; ni++) {
+    const int64_t n = (int64_t)no * wpt + ni;
+    if (n >= N) break;
+    const int64_t id0 = n * D + (int64_t)c8 * 8;
+    const vec8 x = stream_load(reinterpret_cast<const vec8*>(data + id0));
+    const T lo = mn[n], sc = scale[n];
+    float u[8];
+    if (NOISE == GACT_NOISE_INJECT) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(noise + id0), b = *reinterpret_cast<const f32x4*>(noise + id0 + 4);
+      u[0] = a.x; u[1] = a.y; u[2] = a.z; u[3] = a.w; u[4] = b.x; u[5] = b.y; u[6] = b.z; u[7] = b.w;
+    } else if (NOISE == GACT_NOISE_REF) {
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const uint64_t j = (uint64_t)(j0 + e);
+        if ((ni & 3) == 0) philox4x32_10(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r[e]);
+        u[e] = curand_uniform_map(r[e][ni & 3]);
+      }
+    } else if (NOISE == GACT_NOISE_FAST) {
+      const uint64_t blk = (uint64_t)id0 >> 3;
+      philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r[0]);
+#pragma unroll
+      for (int e = 0; e < 8; e++) u[e] = fast_uniform_map((e & 1) ? (r[0][e >> 1] >> 16) : (r[0][e >> 1] & 0xffffu));
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; e++) u[e] = 0.5f;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      typename Elem<T>::Store one;
+      Elem<T>::set(one, 0, 0, x[e]);
+      bytes[e] |= Elem<T>::code1(one, 0, 0, lo, sc, u[e]) << (ni * bits);
+    }
+  }
+  u32x2 w;
+  w.x = (bytes[0] & 0xffu) | ((bytes[1] & 0xffu) << 8) | ((bytes[2] & 0xffu) << 16) | (bytes[3] << 24);
+  w.y = (bytes[4] & 0xffu) | ((bytes[5] & 0xffu) << 8) | ((bytes[6] & 0xffu) << 16) | (bytes[7] << 24);
+  stream_store(w, reinterpret_cast<u32x2*>(packed + j0));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+unpack_rows8_kernel(const uint8_t* __restrict__ packed, int bits, const T* __restrict__ scale,
+                    const T* __restrict__ mn, int64_t N, uint32_t tpr, uint32_t total_threads, T* __restrict__ out) {
+  const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= total_threads) return;
+  const int wpt = 8 / bits;
+  const uint32_t no = t / tpr, c8 = t - no * tpr;
+  const int64_t D = (int64_t)tpr * 8;
+  const u32x2 w = stream_load(reinterpret_cast<const u32x2*>(packed + (int64_t)no * D + (int64_t)c8 * 8));
+  typedef T vec8 __attribute__((ext_vector_type(8)));
+  for (int ni = 0; ni < wpt; ni++) {
+    const int64_t n = (int64_t)no * wpt + ni;
+    if (n >= N) break;
+    const typename Elem<T>::Dq dq = Elem<T>::dq_prepare(scale[n], mn[n]);
+    vec8 v;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const uint32_t byte = ((e < 4 ? w.x : w.y) >> (8 * (e & 3))) & 0xffu;
+      v[e] = Elem<T>::decode((int)((byte >> (ni * bits)) & ((1u << bits) - 1u)), dq);
+    }
+    stream_store(v, reinterpret_cast<vec8*>(out + n * D + (int64_t)c8 * 8));
+  }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Dropout-mask bit packing.  Within each 512-element block, element e = k*16 + w is bit k of word w
 // (quantization_cuda_kernel.cu:228-252): with one 16-byte load per lane, lane k holds elements
@@ -1510,26 +1592,56 @@ void launch_minimax_any(const T* x, int64_t N, int64_t D, T* mn, T* mx, hipStrea
     hipLaunchKernelGGL((minimax_any_kernel<T, false, 1>), grid, block, 0, stream, x, N, D, lpr_log2, mn, mx);
 }
 
+// the 8-columns-per-thread kernels take G = 1, D % 8 == 0, 16-byte aligned rows, and a thread count that fits 32 bits
+inline bool rows8_ok(int bits, int64_t N, int64_t G, int64_t D, uint32_t* tpr, uint32_t* total) {
+  if (G != 1 || D % 8 != 0 || D / 8 > 0x7fffffffLL) return false;
+  const int64_t rows = supergroups(N, bits), threads = rows * (D / 8);
+  if (threads <= 0 || threads > 0xffffff00LL) return false;
+  *tpr = (uint32_t)(D / 8);
+  *total = (uint32_t)threads;
+  return true;
+}
+
 template <typename T>
 int pack_any(const T* data, const T* mn, const T* scale, int bits, int64_t N, int64_t G, int64_t D, int noise_mode,
              uint64_t seed, const float* noise, uint8_t* packed, hipStream_t stream) {
+  uint32_t tpr = 0, threads = 0;
+  const bool rows8 = rows8_ok(bits, N, G, D, &tpr, &threads) && aligned16(data) && aligned16(packed) &&
+                     (D * (int64_t)sizeof(T)) % 16 == 0 && (noise_mode != GACT_NOISE_INJECT || aligned16(noise));
   const int64_t total = gact_packed_bytes(bits, N, G, D);
-  const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  const dim3 grid((unsigned)(rows8 ? (threads + 255u) / 256u : (total + 255) / 256)), block(256);
+#define GACT_LAUNCH_PACK(M)                                                                                          \
+  do {                                                                                                               \
+    if (rows8)                                                                                                       \
+      hipLaunchKernelGGL((pack_rows8_kernel<T, M>), grid, block, 0, stream, data, mn, scale, bits, N, tpr, threads,   \
+                         seed, noise, packed);                                                                       \
+    else                                                                                                             \
+      hipLaunchKernelGGL((pack_any_kernel<T, M>), grid, block, 0, stream, data, mn, scale, bits, N, G, D, seed,       \
+                         noise, packed, total);                                                                      \
+  } while (0)
   switch (noise_mode) {
-    case GACT_NOISE_CONST:
-      hipLaunchKernelGGL((pack_any_kernel<T, GACT_NOISE_CONST>), grid, block, 0, stream, data, mn, scale, bits, N, G, D, seed, noise, packed, total);
-      break;
-    case GACT_NOISE_INJECT:
-      hipLaunchKernelGGL((pack_any_kernel<T, GACT_NOISE_INJECT>), grid, block, 0, stream, data, mn, scale, bits, N, G, D, seed, noise, packed, total);
-      break;
-    case GACT_NOISE_REF:
-      hipLaunchKernelGGL((pack_any_kernel<T, GACT_NOISE_REF>), grid, block, 0, stream, data, mn, scale, bits, N, G, D, seed, noise, packed, total);
-      break;
-    case GACT_NOISE_FAST:
-      hipLaunchKernelGGL((pack_any_kernel<T, GACT_NOISE_FAST>), grid, block, 0, stream, data, mn, scale, bits, N, G, D, seed, noise, packed, total);
-      break;
-    default:
-      return GACT_EINVAL;
+    case GACT_NOISE_CONST: GACT_LAUNCH_PACK(GACT_NOISE_CONST); break;
+    case GACT_NOISE_INJECT: GACT_LAUNCH_PACK(GACT_NOISE_INJECT); break;
+    case GACT_NOISE_REF: GACT_LAUNCH_PACK(GACT_NOISE_REF); break;
+    case GACT_NOISE_FAST: GACT_LAUNCH_PACK(GACT_NOISE_FAST); break;
+    default: return GACT_EINVAL;
+  }
+#undef GACT_LAUNCH_PACK
+  return launch_status();
+}
+
+template <typename T>
+int unpack_any(const uint8_t* packed, int bits, const T* scale, const T* mn, int64_t N, int64_t G, int64_t D, T* out,
+               hipStream_t stream) {
+  uint32_t tpr = 0, threads = 0;
+  if (rows8_ok(bits, N, G, D, &tpr, &threads) && aligned16(out) && (reinterpret_cast<uintptr_t>(packed) & 7u) == 0 &&
+      (D * (int64_t)sizeof(T)) % 16 == 0) {
+    hipLaunchKernelGGL((unpack_rows8_kernel<T>), dim3((threads + 255u) / 256u), dim3(256), 0, stream, packed, bits, scale,
+                       mn, N, tpr, threads, out);
+  } else {
+    const int64_t total = gact_packed_bytes(bits, N, G, D);
+    hipLaunchKernelGGL((unpack_any_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, packed, bits,
+                       scale, mn, N, G, D, out, total);
   }
   return launch_status();
 }
@@ -1622,13 +1734,9 @@ int gact_unpack(const void* packed, int bits, const void* scale, const void* mn,
       return dispatch_dequantize<float>(bits, (const uint8_t*)packed, (const float*)scale, (const float*)mn, N * GROUP, N, (float*)out, s);
     return dispatch_dequantize<f16>(bits, (const uint8_t*)packed, (const f16*)scale, (const f16*)mn, N * GROUP, N, (f16*)out, s);
   }
-  const int64_t total = gact_packed_bytes(bits, N, G, D);
-  const dim3 grid((unsigned)((total + 255) / 256)), block(256);
   if (dtype == GACT_F32)
-    hipLaunchKernelGGL((unpack_any_kernel<float>), grid, block, 0, s, (const uint8_t*)packed, bits, (const float*)scale, (const float*)mn, N, G, D, (float*)out, total);
-  else
-    hipLaunchKernelGGL((unpack_any_kernel<f16>), grid, block, 0, s, (const uint8_t*)packed, bits, (const f16*)scale, (const f16*)mn, N, G, D, (f16*)out, total);
-  return launch_status();
+    return unpack_any<float>((const uint8_t*)packed, bits, (const float*)scale, (const float*)mn, N, G, D, (float*)out, s);
+  return unpack_any<f16>((const uint8_t*)packed, bits, (const f16*)scale, (const f16*)mn, N, G, D, (f16*)out, s);
 }
 
 int gact_quantize(const void* x, int dtype, int64_t numel, int bits, int noise_mode, uint64_t seed, const float* noise,

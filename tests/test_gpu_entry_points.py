@@ -49,7 +49,8 @@ def test_minimax_on_a_base_address_that_is_not_16_byte_aligned(dtype, shape):
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f16"])
 @pytest.mark.parametrize("bits", [1, 2, 4, 8])
-@pytest.mark.parametrize("ngd", [(203, 1, 256), (21, 3, 64), (10, 2, 256), (9, 1, 128)])
+@pytest.mark.parametrize("ngd", [(203, 1, 256), (21, 3, 64), (10, 2, 256), (9, 1, 128), (33, 1, 64), (5, 1, 1024),
+                                 (12, 1, 96), (7, 1, 72), (6, 1, 100)])
 @pytest.mark.parametrize("stream", ["deterministic", "reference", "fast"])
 def test_pack_unpack_entry_points(dtype, bits, ngd, stream):
     N, G, D = ngd
