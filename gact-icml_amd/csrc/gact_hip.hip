@@ -1416,12 +1416,13 @@ quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_
                         uint8_t* __restrict__ min_arena) {
   // the plan did not fit the arena or held an invalid width, or no tensor has this width
   if (plan[1] == 0 || plan[2 + (BITS == 1 ? 0 : BITS == 2 ? 1 : BITS == 4 ? 2 : 3)] == 0) return;
-  const int t = block_map ? block_map[blockIdx.x] : batch_find(table, L, blockIdx.x);
+  const int64_t block = blockIdx.x;  // the XCD-aware order gains nothing here (800 -> 797 us on 120 half tensors)
+  const int t = block_map ? block_map[block] : batch_find(table, L, block);
   if (bits[t] != BITS) return;
   const gact_batch_entry ent = table[t];
   if (ent.dtype != (sizeof(T) == 4 ? GACT_F32 : GACT_F16)) return;
   const int64_t N = (ent.numel + GROUP - 1) / GROUP;
-  const int64_t lb = (int64_t)blockIdx.x - ent.first_block;
+  const int64_t lb = block - ent.first_block;
   quantize_block128<T, BITS, NOISE>((const T*)ent.x, ent.numel, N, lb, packed_arena + ent.packed_offset,
                                     (T*)(scale_arena + ent.stats_offset * 4), (T*)(min_arena + ent.stats_offset * 4),
                                     ent.seed);
@@ -1445,8 +1446,10 @@ dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int3
                           const uint8_t* __restrict__ packed_arena, const uint8_t* __restrict__ scale_arena,
                           const uint8_t* __restrict__ min_arena) {
   if (plan[1] == 0) return;
-  const int64_t block = blockIdx.x >> 1;
-  const int half = blockIdx.x & 1;
+  // half a block is the single-tensor kernel's tile; same XCD-aware order (715 -> 709 us on 120 half tensors)
+  const uint32_t tile = xcd_tile<GACT_XCD_RUN_DQ>(blockIdx.x, gridDim.x);
+  const int64_t block = tile >> 1;
+  const int half = tile & 1;
   const int t = block_map ? block_map[block] : batch_find(table, L, block);
   const gact_batch_entry ent = table[t];
   const int64_t lb = block - ent.first_block;
