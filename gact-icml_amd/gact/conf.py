@@ -29,6 +29,11 @@ class QuantizationConfig:
         self.swap = False
         self.prefetch = False
 
+        # ---- bool masks (not in the reference) ----
+        # Current PyTorch saves dropout masks (and comparison masks) as bool, one byte per element, which the
+        # reference's uint8 rule never sees.  They are packed to one bit per element, losslessly.
+        self.compress_bool_masks = True
+
         # ---- stochastic-rounding noise (not in the reference) ----
         # "fast":          one Philox4x32-10 block per 8 elements, 16-bit uniforms
         # "reference":     the reference's stream (one Philox state per output byte, cuRAND uniform map)

@@ -38,8 +38,10 @@ class Controller:
         self.iter = 0
         self.quantizer = Quantizer(default_bit=default_bit_for(config.bit), swap=config.swap,
                                    prefetch=config.prefetch)
-        # parameters are saved for backward too, and must stay exact
+        # parameters are saved for backward too, and must stay exact; buffers (running statistics, constant
+        # masks) live as long as the model, so a packed copy of one would only add memory
         self.quantizer.filter_tensors(model.named_parameters())
+        self.quantizer.filter_tensors(model.named_buffers())
         self.auto_prec = config.auto_prec
         if self.auto_prec:
             self.ap = AutoPrecision(model, self.quantizer, config.bit, config.max_bit, config.work_dir,

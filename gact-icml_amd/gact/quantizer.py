@@ -13,6 +13,7 @@ from .utils import sampled_key_with_sum
 _COMPRESSIBLE = (torch.float32, torch.float16)
 _RANKS = (2, 3, 4)
 KEY_SAMPLES = 100
+BOOL_MASK_MIN_ELEMENTS = 4096     # smaller bool tensors are not worth a kernel launch
 
 
 class _Swap:
@@ -71,13 +72,18 @@ class Quantizer:
     def check_quantize(self, input_tensor):
         """-> (compress?, is it a 0/1 mask?).  The rules of quantizer.py:47-69 in their order: parameters stay;
         a non-empty uint8 tensor is a mask if it holds exactly the values 0 and 1 and is left alone otherwise;
-        then float16/float32 only, requires_grad only (batch-norm statistics do not), rank 2 to 4 only."""
+        then float16/float32 only, requires_grad only (batch-norm statistics do not), rank 2 to 4 only.
+        One rule more than the reference has: a bool tensor on the GPU is a mask by construction (no
+        values to inspect, no synchronisation) when config.compress_bool_masks is set."""
         t = input_tensor
         if t.data_ptr() in self.unrelated_tensors:
             return False, False
         if t.dtype == torch.uint8 and t.numel() > 0:
             lo, hi = torch.aminmax(t)                 # one reduction and one synchronisation for both ends
             is_mask = (int(lo), int(hi)) == (0, 1)
+            return is_mask, is_mask
+        if t.dtype == torch.bool:
+            is_mask = config.compress_bool_masks and t.is_cuda and t.numel() >= BOOL_MASK_MIN_ELEMENTS
             return is_mask, is_mask
         ok = t.dtype in _COMPRESSIBLE and t.requires_grad is not False and t.dim() in _RANKS
         return ok, False
@@ -96,11 +102,14 @@ class Quantizer:
 
     # ---- pack hook ----
     def quantize(self, input):
-        """(False, tensor) when left alone, (True, True, q_mask) for a mask, else (True, False, key, shape, tid)."""
+        """(False, tensor) when left alone, (True, True, q_mask) for a mask (a bool mask adds its dtype as a
+        fourth entry), else (True, False, key, shape, tid)."""
         wanted, is_mask = self.check_quantize(input)
         if not wanted:
             return False, input
         if is_mask:
+            if input.dtype == torch.bool:     # same bytes as a uint8 0/1 mask
+                return True, True, op_quantize_mask(input.view(torch.uint8)), torch.bool
             return True, True, op_quantize_mask(input)
 
         tid = self.tid
@@ -128,7 +137,8 @@ class Quantizer:
         if not input[0]:
             return input[1]
         if input[1]:
-            return op_dequantize_mask(input[2])
+            mask = op_dequantize_mask(input[2])
+            return mask.view(input[3]) if len(input) > 3 else mask
         key, shape, tid = input[2:]
         held = self.ptr_qtensor_map[key]
         q_inputs = held[0]

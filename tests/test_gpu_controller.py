@@ -206,3 +206,56 @@ def test_saved_uint8_mask_takes_the_one_bit_mask_kernels(monkeypatch):
     # the mask comes back exactly; the only lossy tensor is the 8-bit input of the linear layer
     assert torch.equal(lin.bias.grad, mask.float().sum(0))
     assert ((lin.weight.grad - exact).norm() / exact.norm()).item() < 0.02
+
+
+def test_saved_bool_masks_are_packed_to_one_bit_losslessly(monkeypatch):
+    """Not in the reference: dropout in current PyTorch saves a bool mask, which the uint8 rule never sees.
+    With config.compress_bool_masks it goes through the mask kernels (no values inspected, nothing
+    synchronised) and comes back as the same bool tensor, so a dropout layer's gradient is exact."""
+    import gact.quantizer as quantizer_mod
+
+    packed_words = []
+    real_qm = quantizer_mod.op_quantize_mask
+
+    def qm(t):
+        assert t.dtype == torch.uint8
+        q = real_qm(t)
+        packed_words.append(q[0].numel())
+        return q
+
+    monkeypatch.setattr(quantizer_mod, "op_quantize_mask", qm)
+    drop = nn.Dropout(0.3).cuda().train()
+    x = torch.randn(64, 1000, device="cuda", requires_grad=True)
+    upstream = torch.randn(64, 1000, device="cuda")
+
+    def run(hooked):
+        torch.manual_seed(5)
+        torch.cuda.manual_seed_all(5)
+        x.grad = None
+        gact.set_optimization_level("L1")
+        ctl = Controller(drop)
+        if hooked:
+            ctl.install_hook()
+        try:
+            drop(x).backward(upstream)
+        finally:
+            ctl.uninstall_hook()
+        return x.grad.clone()
+
+    exact = run(False)
+    assert packed_words == []
+    assert torch.equal(run(True), exact)
+    assert packed_words == [(64000 + 31) // 32]
+
+    # the tuple protocol: a fourth entry carries the dtype; strided and small tensors
+    q = quantizer_mod.Quantizer(default_bit=4, swap=False, prefetch=False)
+    m = torch.rand(300, 130, device="cuda") < 0.5
+    for t in (m, m.t(), m[::2, 1::3].repeat(3, 5)):
+        h = q.quantize(t)
+        assert h[:2] == (True, True) and h[3] == torch.bool
+        back = q.dequantize(h)
+        assert back.dtype == torch.bool and back.shape == t.shape and torch.equal(back, t)
+    small = torch.rand(10, 10, device="cuda") < 0.5
+    assert q.quantize(small) == (False, small) or q.quantize(small)[1] is small
+    config.compress_bool_masks = False
+    assert q.quantize(m)[0] is False

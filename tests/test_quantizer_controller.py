@@ -51,6 +51,7 @@ def test_filter_rules(rec):
     assert q.check_quantize(torch.tensor([0, 1, 1, 0], dtype=torch.uint8)) == (True, True)   # dropout mask
     assert q.check_quantize(torch.tensor([0, 2, 1, 0], dtype=torch.uint8)) == (False, False)
     assert q.check_quantize(torch.zeros(4, dtype=torch.uint8)) == (False, False)
+    assert q.check_quantize(torch.ones(8192, dtype=torch.bool)) == (False, False)   # bool masks: only on the GPU
 
 
 def test_tuple_protocol_tids_seeds_and_tables(rec):
