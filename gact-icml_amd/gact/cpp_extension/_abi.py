@@ -92,13 +92,22 @@ def stream_of(t):
     return torch._C._cuda_getCurrentRawStream(t.device.index)
 
 
+_ONE_GPU = None
+
+
 def call_on(device, fn, *args):
     """Call a library entry point with `device` current (the kernels launch on the current HIP device) and
     turn its status into RuntimeError.  With a single visible GPU there is nothing to switch."""
-    if torch.cuda.device_count() == 1:
-        return check(fn(*args))
-    with torch.cuda.device(device):
-        return check(fn(*args))
+    global _ONE_GPU
+    if _ONE_GPU is None:
+        _ONE_GPU = torch.cuda.device_count() == 1
+    if _ONE_GPU:
+        code = fn(*args)
+    else:
+        with torch.cuda.device(device):
+            code = fn(*args)
+    if code != 0:
+        check(code)
 
 
 def ptr(t):

@@ -55,25 +55,32 @@ def no_scheme_quantize_pack(input, q_bit, seed, *, noise=None, rng_stream=None):
 
     if not input.is_cuda:
         raise RuntimeError("data must be a CUDA tensor!")
-    if input.dtype not in (torch.float32, torch.float16):
+    dtype = input.dtype
+    if dtype is not torch.float32 and dtype is not torch.float16:
         raise RuntimeError("The type of data is not correct!")
     ext_quantization._check_bits(q_bit)
     seed = ext_quantization._seed_u64(seed)
-    x = input.contiguous()  # the reference's reshape copies a non-contiguous input as well
-    if not _abi.aligned(x):
+    # the reference's reshape copies a non-contiguous input as well
+    x = input if input.is_contiguous() else input.contiguous()
+    if x.data_ptr() & 15:
         x = x.clone()
-    mode = ext_quantization._noise_mode(noise, rng_stream)
-    if noise is not None:
-        if (not noise.is_cuda) or noise.dtype != torch.float32 or noise.numel() != N * config.group_size \
-                or not noise.is_contiguous():
-            raise RuntimeError("noise must be a contiguous float32 CUDA tensor with one value per padded element")
-    q_input = torch.empty((ext_quantization.packed_numel(q_bit, N, 1, config.group_size),),
-                          dtype=torch.int8, device=x.device)
-    q_scale = torch.empty((N, 1, 1), dtype=x.dtype, device=x.device)
-    q_min = torch.empty((N, 1, 1), dtype=x.dtype, device=x.device)
-    _abi.call_on(x.device, _abi.lib().gact_quantize, x.data_ptr(), _abi.dtype_code(x.dtype), x.numel(), q_bit, mode,
-                 seed, _abi.ptr(noise), q_input.data_ptr(), q_scale.data_ptr(), q_min.data_ptr(), None,
-                 _abi.stream_of(x))
+    if noise is None and rng_stream is None:
+        mode = _abi.NOISE_MODES.get(config.rng_stream)
+        if mode is None:
+            mode = ext_quantization._noise_mode(None, None)      # raises, naming the streams there are
+    else:
+        mode = ext_quantization._noise_mode(noise, rng_stream)
+        if noise is not None:
+            if (not noise.is_cuda) or noise.dtype != torch.float32 or noise.numel() != N * config.group_size \
+                    or not noise.is_contiguous():
+                raise RuntimeError("noise must be a contiguous float32 CUDA tensor with one value per padded element")
+    device = x.device
+    q_input = torch.empty(ext_quantization.packed_numel(q_bit, N, 1, _abi.GROUP), dtype=torch.int8, device=device)
+    q_scale = torch.empty((N, 1, 1), dtype=dtype, device=device)
+    q_min = torch.empty((N, 1, 1), dtype=dtype, device=device)
+    _abi.call_on(device, _abi.lib().gact_quantize, x.data_ptr(), _abi.F32 if dtype is torch.float32 else _abi.F16,
+                 x.numel(), q_bit, mode, seed, None if noise is None else noise.data_ptr(), q_input.data_ptr(),
+                 q_scale.data_ptr(), q_min.data_ptr(), None, torch._C._cuda_getCurrentRawStream(device.index))
     return q_input, q_scale, q_min
 
 
@@ -126,16 +133,17 @@ def op_dequantize(input, input_shape):
     ext_quantization._check_bits(q_bit)
     if not q_input.is_cuda:
         raise RuntimeError("data must be a CUDA tensor!")
-    if q_input.dtype != torch.int8 or q_input.dim() != 1:
+    if q_input.dtype is not torch.int8 or q_input.dim() != 1:
         raise RuntimeError("The type of data is not correct!")
     N = _num_groups(num_features)
-    if q_input.numel() < ext_quantization.packed_numel(q_bit, N, 1, config.group_size) - 1 \
+    if q_input.numel() < ext_quantization.packed_numel(q_bit, N, 1, _abi.GROUP) - 1 \
             or q_scale.numel() < N or q_min.numel() < N:
         raise RuntimeError("packed data / scale / min are too short for shape %s" % (tuple(input_shape),))
-    if q_scale.dtype != q_min.dtype:
+    dtype = q_scale.dtype
+    if dtype is not q_min.dtype:
         raise RuntimeError("expected scalar type of min to match scale")
-    out = torch.empty(tuple(input_shape), dtype=q_scale.dtype, device=q_input.device)
-    _abi.call_on(q_input.device, _abi.lib().gact_dequantize, q_input.data_ptr(), q_bit, q_scale.data_ptr(),
-                 q_min.data_ptr(), _abi.dtype_code(q_scale.dtype), num_features, out.data_ptr(),
-                 _abi.stream_of(q_input))
+    device = q_input.device
+    out = torch.empty(tuple(input_shape), dtype=dtype, device=device)
+    _abi.call_on(device, _abi.lib().gact_dequantize, q_input.data_ptr(), q_bit, q_scale.data_ptr(), q_min.data_ptr(),
+                 _abi.dtype_code(dtype), num_features, out.data_ptr(), torch._C._cuda_getCurrentRawStream(device.index))
     return out
