@@ -132,6 +132,15 @@ def test_config3_bert_large_fp16(name, shape, kind, bits):
     cross_check_kernel_paths(x, q, bits, "fast", 7)
 
 
+@pytest.mark.parametrize("dtype,bits", [(torch.float16, 8), (torch.float32, 1), (torch.float32, 8)])
+def test_launches_with_capped_occupancy(dtype, bits):
+    """From 196 608 groups on some kernels are launched with fewer resident waves per CU (a request for dynamic
+    LDS that they never touch): the widths and types whose capped launch no BASELINE workload reaches."""
+    x = gen((196608 + 3, 256), dtype, "relu", 5)
+    q, out = check_against_oracle(x, bits, "fast", 13)
+    check_properties(x, q, out, bits, stochastic=True)
+
+
 def test_config4_gcn_features_fp32_1bit():
     x = gen((169343, 256), torch.float32, "relu60", 4)
     zeros = (x == 0).float().mean().item()
