@@ -268,3 +268,42 @@ def test_batched_refuses_an_arena_that_is_too_small():
     q = bq.quantize(tensors, bits, [0, 1, 2], arena_bytes=1 << 20)
     ok, need = q.ok()
     assert not ok and need == 3 * 4096 * 256
+
+
+def test_random_cases_on_general_shapes_masks_and_minimax():
+    """600 seeded random cases on what the fixed parametrisations above only sample: (N, G, D) of any kind
+    through pack / unpack, masks of any length, minimax on any row length and alignment."""
+    rng = np.random.default_rng(2024)
+    modes = {"deterministic": 0, "reference": 2, "fast": 3}
+    for case in range(600):
+        kind = case % 3
+        dtype = DTYPES[int(rng.integers(0, 2))]
+        if kind == 0:
+            N, G = int(rng.integers(1, 60)), int(rng.integers(1, 4))
+            D = int(rng.choice([8, 24, 40, 64, 100, 128, 256, 264, 512]))
+            bits, stream, seed = int(rng.choice([1, 2, 4, 8])), str(rng.choice(list(modes))), int(rng.integers(0, 2 ** 31 - 1))
+            x = torch.randn((N, G, D), generator=torch.Generator().manual_seed(case)).to(dtype)
+            rows = x.reshape(N * G, D)
+            mn_np, mx_np = rows.min(1).values.numpy(), rows.max(1).values.numpy()
+            sc_np = oracle.scale(mn_np, mx_np, bits)
+            want = oracle.pack(x.numpy(), mn_np, sc_np, bits, modes[stream], seed)
+            mn = torch.from_numpy(mn_np).reshape(N, G, 1).cuda()
+            mx = torch.from_numpy(mx_np).reshape(N, G, 1).cuda()
+            packed, scale = ext_quantization.pack_single_precision(x.cuda(), mn, mx, bits, True, seed, rng_stream=stream)
+            tag = "case %d: %s N=%d G=%d D=%d bits=%d %s" % (case, dtype, N, G, D, bits, stream)
+            np.testing.assert_array_equal(packed.cpu().numpy().view(np.uint8)[:want.size], want, err_msg=tag)
+            out = ext_quantization.unpack_single_precision(packed, bits, scale, mn, N, G, D)
+            ref = oracle.unpack(want, bits, sc_np, mn_np, N, G, D)
+            np.testing.assert_array_equal(bits_view(out.cpu().numpy().reshape(-1)), bits_view(ref.reshape(-1)), err_msg=tag)
+        elif kind == 1:
+            n = int(rng.integers(1, 70000))
+            data = (torch.rand(n, generator=torch.Generator().manual_seed(case)) < float(rng.random())).to(torch.uint8)
+            q = ops.op_quantize_mask(data.cuda())
+            np.testing.assert_array_equal(q[0].cpu().numpy(), oracle.mask_pack(data.numpy()), err_msg="mask n=%d" % n)
+            assert torch.equal(ops.op_dequantize_mask(q).cpu(), data), n
+        else:
+            N, D, off = int(rng.integers(1, 300)), 32 * int(rng.integers(2, 80)), int(rng.integers(0, 2))
+            buf = torch.randn(N * D + off, generator=torch.Generator().manual_seed(case)).to(dtype).cuda()
+            x = buf[off:].view(N, D)
+            mn, mx = ext_minimax.minimax(x)
+            assert torch.equal(mn, x.min(1).values) and torch.equal(mx, x.max(1).values), (N, D, off, dtype)
