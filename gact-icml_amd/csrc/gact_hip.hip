@@ -32,6 +32,7 @@
 #include "gact_hip.h"
 
 typedef _Float16 f16;
+typedef __bf16 bf16;
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
@@ -155,6 +156,10 @@ template <> struct Elem<float> {
   // quantize layout: 4 chunks of 4 columns, 4i + 64m: one 16-byte load per chunk, 256 contiguous
   // bytes per row and load instruction
   static constexpr int kQChunks = 4, kQWidth = 4;
+  static constexpr int kDtype = GACT_F32;
+  typedef float Stat;   // type min, max and scale are computed and stored in (scale: always; min: as T)
+  __device__ static __forceinline__ float stat_of(float x) { return x; }
+  __device__ static __forceinline__ float elem_of(float x) { return x; }
   struct Store { float v[4][4]; };
   __device__ static __forceinline__ void load_noise(const float* p, float (&u)[4]) {
     f32x4 a = stream_load(reinterpret_cast<const f32x4*>(p));
@@ -234,6 +239,10 @@ template <> struct Elem<float> {
 template <> struct Elem<f16> {
   // quantize layout: 2 chunks of 8 columns, 8i + 128m: one 16-byte load per chunk
   static constexpr int kQChunks = 2, kQWidth = 8;
+  static constexpr int kDtype = GACT_F16;
+  typedef f16 Stat;
+  __device__ static __forceinline__ f16 stat_of(f16 x) { return x; }
+  __device__ static __forceinline__ f16 elem_of(f16 x) { return x; }
   struct Store { f16x2 v[2][4]; };   // pairs, so that subtraction and product run as packed ops
   __device__ static __forceinline__ void store_codes(uint8_t* p, const uint32_t (&b)[8]) {
     u32x2 w;
@@ -362,6 +371,72 @@ template <> struct Elem<f16> {
   }
 };
 
+// bfloat16 (not in the reference, which knows float and half): every bfloat16 is a float, so the group is
+// widened on load and quantized exactly as the float path quantizes those floats - same min, same float
+// scale, same codes - with the half layout (8-column chunks, one 16-byte load each).  The scale is kept in
+// float (8 significant bits would not do), the minimum is one of the inputs and goes back to bfloat16
+// unchanged, and dequantize rounds float(code) / scale + min to bfloat16 once, to nearest even.
+template <> struct Elem<bf16> {
+  static constexpr int kQChunks = 2, kQWidth = 8;
+  static constexpr int kDtype = GACT_BF16;
+  typedef float Stat;
+  __device__ static __forceinline__ float stat_of(bf16 x) { return (float)x; }
+  __device__ static __forceinline__ bf16 elem_of(float x) { return (bf16)x; }
+  struct Store { float v[2][8]; };
+  __device__ static __forceinline__ void store_codes(uint8_t* p, const uint32_t (&b)[8]) { Elem<f16>::store_codes(p, b); }
+  __device__ static __forceinline__ void load_noise(const float* p, float (&u)[8]) { Elem<f16>::load_noise(p, u); }
+  __device__ static __forceinline__ void load_chunk(const bf16* p, Store& st, int k) {
+    const u32x4 a = stream_load(reinterpret_cast<const u32x4*>(p));
+    const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      st.v[k][2 * j] = __builtin_bit_cast(float, w[j] << 16);
+      st.v[k][2 * j + 1] = __builtin_bit_cast(float, w[j] & 0xffff0000u);
+    }
+  }
+  __device__ static __forceinline__ void set(Store& st, int k, int e, bf16 x) { st.v[k][e] = (float)x; }
+  __device__ static __forceinline__ void group_minmax(const Store& st, float& lo_out, float& hi_out) {
+    float lo = Elem<float>::init_lo(), hi = Elem<float>::init_hi();
+#pragma unroll
+    for (int k = 0; k < 2; k++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        lo = __builtin_fminf(lo, st.v[k][e]);
+        hi = __builtin_fmaxf(hi, st.v[k][e]);
+      }
+    row_all_minmax(lo, hi);
+    lo_out = lo;
+    hi_out = hi;
+  }
+  __device__ static __forceinline__ float make_scale(float lo, float hi, int qmax) {
+    return Elem<float>::make_scale(lo, hi, qmax);
+  }
+  __device__ static __forceinline__ uint32_t code1(const Store& st, int k, int e, float mn, float s, float u) {
+    float t = st.v[k][e] - mn;
+    float y = __builtin_fmaf(t, s, u);
+    return rint_clamp0(y - 0.5f);
+  }
+  template <bool CONST_NOISE>
+  __device__ static __forceinline__ void codes(const Store& st, int k, float mn, float s, const float (&u)[8],
+                                               uint32_t (&c)[8]) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) c[e] = code1(st, k, e, mn, s, u[e]);
+  }
+  __device__ static __forceinline__ bf16 finish(float q, float mn) { return (bf16)(q + mn); }
+  __device__ static __forceinline__ uint32_t table_entry(float c, float s, float mn) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (bf16)(c / s + mn));
+  }
+  __device__ static __forceinline__ bf16 from_bits(uint32_t b) { return __builtin_bit_cast(bf16, (uint16_t)b); }
+  static constexpr int kDqWidth = 8;
+  __device__ static __forceinline__ void store_dq(bf16* p, const bf16 (&v)[8]) {
+    typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+    bf16x8 a;
+#pragma unroll
+    for (int e = 0; e < 8; e++) a[e] = v[e];
+    stream_store(a, reinterpret_cast<bf16x8*>(p));
+  }
+};
+
 // Column of the first element of chunk k for row lane i: chunks are W columns wide and 16*W apart.
 template <typename T>
 __device__ __forceinline__ int chunk_col(int k, int i) { return Elem<T>::kQWidth * (16 * k + i); }
@@ -382,7 +457,7 @@ __device__ __forceinline__ void load_group(const T* __restrict__ x, int64_t nume
 #pragma unroll
       for (int e = 0; e < W; e++) {
         int64_t idx = base + chunk_col<T>(k, i) + e;
-        Elem<T>::set(st, k, e, idx < numel ? x[idx] : (T)0);
+        Elem<T>::set(st, k, e, idx < numel ? x[idx] : (T)0.0f);
       }
   }
 }
@@ -456,7 +531,8 @@ __device__ __forceinline__ void fast_noise(int64_t n, int i, uint32_t k0, uint32
 // ------------------------------------------------------------------------------------------------
 template <typename T, int BITS, int NOISE, bool GIVEN>
 __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int64_t numel, int64_t N, int64_t sg,
-                                                    int i, uint8_t* __restrict__ packed, T* __restrict__ scale_out,
+                                                    int i, uint8_t* __restrict__ packed,
+                                                    typename Elem<T>::Stat* __restrict__ scale_out,
                                                     T* mn_io, T* mx_io, uint32_t k0, uint32_t k1,
                                                     const float* __restrict__ noise) {
   constexpr int WPT = 8 / BITS;
@@ -465,7 +541,8 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
   const int64_t n0 = sg * WPT;
 
   typename Elem<T>::Store v[WPT];
-  T lo_t[WPT], hi_t[WPT], s_t[WPT];
+  typedef typename Elem<T>::Stat Stat;
+  Stat lo_t[WPT], hi_t[WPT], s_t[WPT];
 #pragma unroll
   for (int ni = 0; ni < WPT; ni++) {
     if (n0 + ni < N) load_group<T>(x, numel, n0 + ni, i, v[ni]);
@@ -473,12 +550,12 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
 #pragma unroll
   for (int ni = 0; ni < WPT; ni++) {
     const int64_t n = n0 + ni;
-    lo_t[ni] = (T)0;
-    hi_t[ni] = (T)0;
+    lo_t[ni] = (Stat)0.0f;
+    hi_t[ni] = (Stat)0.0f;
     if (n < N) {
       if (GIVEN) {
-        lo_t[ni] = mn_io[n];
-        hi_t[ni] = mx_io[n];
+        lo_t[ni] = Elem<T>::stat_of(mn_io[n]);
+        hi_t[ni] = Elem<T>::stat_of(mx_io[n]);
       } else {
         Elem<T>::group_minmax(v[ni], lo_t[ni], hi_t[ni]);
       }
@@ -487,18 +564,18 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
   // one scale division per lane: lane j of the row takes group j % WPT, then the row shares the results
   {
     const int mine = i & (WPT - 1);
-    T lo_m = lo_t[0], hi_m = hi_t[0];
+    Stat lo_m = lo_t[0], hi_m = hi_t[0];
 #pragma unroll
     for (int ni = 1; ni < WPT; ni++) {
       lo_m = (mine == ni) ? lo_t[ni] : lo_m;
       hi_m = (mine == ni) ? hi_t[ni] : hi_m;
     }
-    const T s_m = Elem<T>::make_scale(lo_m, hi_m, QMAX);
+    const Stat s_m = Elem<T>::make_scale(lo_m, hi_m, QMAX);
     if (i < WPT && n0 + i < N) {
       scale_out[n0 + i] = s_m;
       if (!GIVEN) {
-        mn_io[n0 + i] = lo_m;
-        if (mx_io) mx_io[n0 + i] = hi_m;
+        mn_io[n0 + i] = Elem<T>::elem_of(lo_m);
+        if (mx_io) mx_io[n0 + i] = Elem<T>::elem_of(hi_m);
       }
     }
     if (WPT == 1) {
@@ -595,9 +672,11 @@ __device__ __forceinline__ float row_bcast_at(float v, int g) {
 }
 
 template <typename T, int BITS, int SGS>
-__device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
+__device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ packed,
+                                                const typename Elem<T>::Stat* __restrict__ scale,
                                                 const T* __restrict__ mn, int64_t numel, int64_t N, int64_t unit,
                                                 int l, T* __restrict__ out) {
+  typedef typename Elem<T>::Stat Stat;
   constexpr int WPT = 8 / BITS;
   constexpr int W = Elem<T>::kDqWidth;
   constexpr int G = SGS * WPT;
@@ -635,7 +714,8 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
       const int e = p * LPU + l;
       const int64_t g = g0 + e / ENT;
       const bool live = e < TOT && g < N;
-      tab[p] = Elem<T>::table_entry((float)(e & (ENT - 1)), live ? scale[g] : (T)1, live ? mn[g] : (T)0);
+      tab[p] = Elem<T>::table_entry((float)(e & (ENT - 1)), live ? scale[g] : (Stat)1.0f,
+                                    live ? Elem<T>::stat_of(mn[g]) : (Stat)0.0f);
     }
     const uint32_t unitbase = (threadIdx.x & 63u) & ~(uint32_t)(LPU - 1);  // first lane of the unit within its wave
 #pragma unroll
@@ -666,26 +746,29 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
     return;
   } else {
   // 8 bit.  scale and min of the unit's groups: 16-byte loads when the whole unit exists and the arrays allow it
-  constexpr int PER16 = 16 / (int)sizeof(T);
-  T sv[G], mv[G];
-  if (G % PER16 == 0 && g0 + G <= N &&
+  constexpr int PERS = 16 / (int)sizeof(Stat), PERM = 16 / (int)sizeof(T);
+  Stat sv[G], mv[G];
+  if (G % PERS == 0 && G % PERM == 0 && g0 + G <= N &&
       ((reinterpret_cast<uintptr_t>(scale + g0) | reinterpret_cast<uintptr_t>(mn + g0)) & 15u) == 0) {
-    typedef T vec16 __attribute__((ext_vector_type(PER16)));
+    typedef Stat svec __attribute__((ext_vector_type(PERS)));
+    typedef T mvec __attribute__((ext_vector_type(PERM)));
 #pragma unroll
-    for (int c = 0; c < G / PER16; c++) {
-      const vec16 a = *reinterpret_cast<const vec16*>(scale + g0 + c * PER16);
-      const vec16 m = *reinterpret_cast<const vec16*>(mn + g0 + c * PER16);
+    for (int c = 0; c < G / PERS; c++) {
+      const svec a = *reinterpret_cast<const svec*>(scale + g0 + c * PERS);
 #pragma unroll
-      for (int e = 0; e < PER16; e++) {
-        sv[c * PER16 + e] = a[e];
-        mv[c * PER16 + e] = m[e];
-      }
+      for (int e = 0; e < PERS; e++) sv[c * PERS + e] = a[e];
+    }
+#pragma unroll
+    for (int c = 0; c < G / PERM; c++) {
+      const mvec m = *reinterpret_cast<const mvec*>(mn + g0 + c * PERM);
+#pragma unroll
+      for (int e = 0; e < PERM; e++) mv[c * PERM + e] = Elem<T>::stat_of(m[e]);
     }
   } else {
 #pragma unroll
     for (int g = 0; g < G; g++) {
-      sv[g] = g0 + g < N ? scale[g0 + g] : (T)1;
-      mv[g] = g0 + g < N ? mn[g0 + g] : (T)0;
+      sv[g] = g0 + g < N ? scale[g0 + g] : (Stat)1.0f;
+      mv[g] = g0 + g < N ? Elem<T>::stat_of(mn[g0 + g]) : (Stat)0.0f;
     }
   }
   // one correctly rounded reciprocal per group and row instead of one per group and lane: row lane j takes
@@ -732,7 +815,8 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
 // rows, so that every pass of the block reads one contiguous stretch.
 template <typename T, int BITS, int NOISE>
 __device__ __forceinline__ void quantize_block128(const T* __restrict__ x, int64_t numel, int64_t N, int64_t lb,
-                                                  uint8_t* __restrict__ packed, T* __restrict__ scale_out,
+                                                  uint8_t* __restrict__ packed,
+                                                  typename Elem<T>::Stat* __restrict__ scale_out,
                                                   T* __restrict__ mn_out, uint64_t seed) {
   constexpr int WPT = 8 / BITS;
   const int row = threadIdx.x >> 4, i = threadIdx.x & 15;
@@ -748,7 +832,8 @@ __device__ __forceinline__ void quantize_block128(const T* __restrict__ x, int64
 // (a wave for float, half a wave for half) gets one unit for half and two for float - several units in a
 // row per wave cost 10-20 %.
 template <typename T, int BITS>
-__device__ __forceinline__ void dequantize_block128(const uint8_t* __restrict__ packed, const T* __restrict__ scale,
+__device__ __forceinline__ void dequantize_block128(const uint8_t* __restrict__ packed,
+                                                    const typename Elem<T>::Stat* __restrict__ scale,
                                                     const T* __restrict__ mn, int64_t numel, int64_t N, int64_t lb,
                                                     int half, T* __restrict__ out) {
   constexpr int LPU = GROUP / Elem<T>::kDqWidth;  // lanes per unit
@@ -813,7 +898,8 @@ __device__ __forceinline__ uint32_t xcd_tile(uint32_t b, uint32_t nb) {
 template <typename T, int BITS, int NOISE, bool GIVEN>
 __global__ void __launch_bounds__(256)
 quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
-                T* __restrict__ scale_out, T* mn_io, T* mx_io, uint64_t seed, const float* __restrict__ noise) {
+                typename Elem<T>::Stat* __restrict__ scale_out, T* mn_io, T* mx_io, uint64_t seed,
+                const float* __restrict__ noise) {
   constexpr uint32_t RUN = BITS >= 4 ? GACT_XCD_RUN_Q : GACT_XCD_RUN_Q_LOW;
   const int64_t sg = (int64_t)xcd_tile<RUN>(blockIdx.x, gridDim.x) * (blockDim.x >> 4) + (threadIdx.x >> 4);
   if (sg * (8 / BITS) >= N) return;
@@ -823,7 +909,8 @@ quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __re
 
 template <typename T, int BITS>
 __global__ void __launch_bounds__(256)
-dequantize_kernel(const uint8_t* __restrict__ packed, const T* __restrict__ scale, const T* __restrict__ mn,
+dequantize_kernel(const uint8_t* __restrict__ packed, const typename Elem<T>::Stat* __restrict__ scale,
+                  const T* __restrict__ mn,
                   int64_t numel, int64_t N, T* __restrict__ out) {
   constexpr int LPU = GROUP / Elem<T>::kDqWidth;  // lanes per unit of 8 groups: 64 (float) or 32 (half)
   const int64_t unit = ((int64_t)xcd_tile<GACT_XCD_RUN_DQ>(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x) / LPU;
@@ -1420,12 +1507,12 @@ quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_
   const int t = block_map ? block_map[block] : batch_find(table, L, block);
   if (bits[t] != BITS) return;
   const gact_batch_entry ent = table[t];
-  if (ent.dtype != (sizeof(T) == 4 ? GACT_F32 : GACT_F16)) return;
+  if (ent.dtype != Elem<T>::kDtype) return;
   const int64_t N = (ent.numel + GROUP - 1) / GROUP;
   const int64_t lb = block - ent.first_block;
   quantize_block128<T, BITS, NOISE>((const T*)ent.x, ent.numel, N, lb, packed_arena + ent.packed_offset,
-                                    (T*)(scale_arena + ent.stats_offset * 4), (T*)(min_arena + ent.stats_offset * 4),
-                                    ent.seed);
+                                    (typename Elem<T>::Stat*)(scale_arena + ent.stats_offset * 4),
+                                    (T*)(min_arena + ent.stats_offset * 4), ent.seed);
 }
 
 // Dequantize, one launch for all widths (every width fits 60 registers): the width of a block's tensor is read
@@ -1436,8 +1523,10 @@ __device__ __forceinline__ void dequantize_batched_block(const gact_batch_entry&
   const int64_t N = (ent.numel + GROUP - 1) / GROUP;
   if (ent.dtype == GACT_F32)
     dequantize_block128<float, BITS>(packed, (const float*)sc, (const float*)mn, ent.numel, N, lb, half, (float*)ent.x);
-  else
+  else if (ent.dtype == GACT_F16)
     dequantize_block128<f16, BITS>(packed, (const f16*)sc, (const f16*)mn, ent.numel, N, lb, half, (f16*)ent.x);
+  else
+    dequantize_block128<bf16, BITS>(packed, (const float*)sc, (const bf16*)mn, ent.numel, N, lb, half, (bf16*)ent.x);
 }
 // grid: two workgroups per block of 128 groups
 __global__ void __launch_bounds__(256)
@@ -1519,7 +1608,8 @@ inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
 }
 
 template <typename T, int BITS, bool GIVEN>
-int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, T* scale, T* mn, T* mx, int noise_mode,
+int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, typename Elem<T>::Stat* scale, T* mn, T* mx,
+                    int noise_mode,
                     uint64_t seed, const float* noise, hipStream_t stream) {
   dim3 grid, block;
   row_grid(supergroups(N, BITS), &grid, &block, quantize_threads(BITS, sizeof(T)));
@@ -1549,7 +1639,8 @@ int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, T* sc
 }
 
 template <typename T, bool GIVEN>
-int dispatch_quantize(int bits, const T* x, int64_t numel, int64_t N, uint8_t* packed, T* scale, T* mn, T* mx,
+int dispatch_quantize(int bits, const T* x, int64_t numel, int64_t N, uint8_t* packed, typename Elem<T>::Stat* scale,
+                      T* mn, T* mx,
                       int noise_mode, uint64_t seed, const float* noise, hipStream_t stream) {
   switch (bits) {
     case 1: return launch_quantize<T, 1, GIVEN>(x, numel, N, packed, scale, mn, mx, noise_mode, seed, noise, stream);
@@ -1561,7 +1652,8 @@ int dispatch_quantize(int bits, const T* x, int64_t numel, int64_t N, uint8_t* p
 }
 
 template <typename T>
-int dispatch_dequantize(int bits, const uint8_t* packed, const T* scale, const T* mn, int64_t numel, int64_t N, T* out,
+int dispatch_dequantize(int bits, const uint8_t* packed, const typename Elem<T>::Stat* scale, const T* mn,
+                        int64_t numel, int64_t N, T* out,
                         hipStream_t stream) {
   // a unit of 8 groups takes 256 / (16 / sizeof(T)) lanes
   const int64_t units_per_block = 256 / (GROUP / (16 / (int64_t)sizeof(T)));
@@ -1746,7 +1838,7 @@ int gact_unpack(const void* packed, int bits, const void* scale, const void* mn,
 
 int gact_quantize(const void* x, int dtype, int64_t numel, int bits, int noise_mode, uint64_t seed, const float* noise,
                   void* packed, void* scale, void* mn, void* mx, void* stream) {
-  if (dtype != GACT_F32 && dtype != GACT_F16) return GACT_EINVAL;
+  if (dtype != GACT_F32 && dtype != GACT_F16 && dtype != GACT_BF16) return GACT_EINVAL;
   if (!valid_bits(bits) || numel < 0) return GACT_EINVAL;
   if (noise_mode < GACT_NOISE_CONST || noise_mode > GACT_NOISE_FAST) return GACT_EINVAL;
   if (numel == 0) return GACT_OK;
@@ -1757,12 +1849,14 @@ int gact_quantize(const void* x, int dtype, int64_t numel, int bits, int noise_m
   hipStream_t s = (hipStream_t)stream;
   if (dtype == GACT_F32)
     return dispatch_quantize<float, false>(bits, (const float*)x, numel, N, (uint8_t*)packed, (float*)scale, (float*)mn, (float*)mx, noise_mode, seed, noise, s);
+  if (dtype == GACT_BF16)
+    return dispatch_quantize<bf16, false>(bits, (const bf16*)x, numel, N, (uint8_t*)packed, (float*)scale, (bf16*)mn, (bf16*)mx, noise_mode, seed, noise, s);
   return dispatch_quantize<f16, false>(bits, (const f16*)x, numel, N, (uint8_t*)packed, (f16*)scale, (f16*)mn, (f16*)mx, noise_mode, seed, noise, s);
 }
 
 int gact_dequantize(const void* packed, int bits, const void* scale, const void* mn, int dtype, int64_t numel, void* out,
                     void* stream) {
-  if (dtype != GACT_F32 && dtype != GACT_F16) return GACT_EINVAL;
+  if (dtype != GACT_F32 && dtype != GACT_F16 && dtype != GACT_BF16) return GACT_EINVAL;
   if (!valid_bits(bits) || numel < 0) return GACT_EINVAL;
   if (numel == 0) return GACT_OK;
   if (!packed || !scale || !mn || !out) return GACT_EINVAL;
@@ -1771,6 +1865,8 @@ int gact_dequantize(const void* packed, int bits, const void* scale, const void*
   hipStream_t s = (hipStream_t)stream;
   if (dtype == GACT_F32)
     return dispatch_dequantize<float>(bits, (const uint8_t*)packed, (const float*)scale, (const float*)mn, numel, N, (float*)out, s);
+  if (dtype == GACT_BF16)
+    return dispatch_dequantize<bf16>(bits, (const uint8_t*)packed, (const float*)scale, (const bf16*)mn, numel, N, (bf16*)out, s);
   return dispatch_dequantize<f16>(bits, (const uint8_t*)packed, (const f16*)scale, (const f16*)mn, numel, N, (f16*)out, s);
 }
 
@@ -1873,6 +1969,10 @@ int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, in
     if (dtypes & GACT_DTYPES_F16) {                                                                           \
       GACT_LAUNCH_QB(f16, 1, M); GACT_LAUNCH_QB(f16, 2, M); GACT_LAUNCH_QB(f16, 4, M);                        \
       GACT_LAUNCH_QB(f16, 8, M);                                                                              \
+    }                                                                                                         \
+    if (dtypes & GACT_DTYPES_BF16) {                                                                          \
+      GACT_LAUNCH_QB(bf16, 1, M); GACT_LAUNCH_QB(bf16, 2, M); GACT_LAUNCH_QB(bf16, 4, M);                     \
+      GACT_LAUNCH_QB(bf16, 8, M);                                                                             \
     }                                                                                                         \
   } while (0)
   switch (noise_mode) {

@@ -1,7 +1,7 @@
 """Training step of a randomly initialised BERT-base classifier with and without activation compression:
 time per iteration and peak device memory per optimisation level.
 
-    python gact-icml_amd/examples/bert_step.py [--batch 16] [--seq 512] [--amp] [--levels L0 L1 L1.2]
+    python gact-icml_amd/examples/bert_step.py [--batch 16] [--seq 512] [--amp | --amp-bf16] [--levels L0 L1 L1.2]
 
 Needs the `transformers` package (no download: the model is built from a default BertConfig).  The usage
 is the reference's: build a Controller on the model, install its hooks, call controller.iterate(backprop)
@@ -19,7 +19,7 @@ import gact  # noqa: E402
 from gact.conf import config  # noqa: E402
 
 
-def run(level, batch, seq, amp, steps):
+def run(level, batch, seq, amp, steps, amp_dtype=torch.float16):
     import transformers
     model_config = transformers.BertConfig()
     model_config._attn_implementation = "eager"
@@ -38,7 +38,7 @@ def run(level, batch, seq, amp, steps):
 
     def backprop():
         model.zero_grad(set_to_none=True)
-        with torch.autocast("cuda", dtype=torch.float16, enabled=amp):
+        with torch.autocast("cuda", dtype=amp_dtype, enabled=amp):
             loss = model(input_ids=ids, labels=labels).loss
         loss.backward()
         return loss
@@ -57,8 +57,9 @@ def run(level, batch, seq, amp, steps):
     if controller is not None:
         controller.uninstall_hook()
     median = sorted(times[2:])[len(times[2:]) // 2]
-    print("%-5s amp=%d batch=%d seq=%d: %6.1f ms/iteration  %6.1f samples/s  peak %5.2f GiB"
-          % (level, amp, batch, seq, median * 1e3, batch / median, torch.cuda.max_memory_allocated() / 2 ** 30), flush=True)
+    mode = "fp32" if not amp else "autocast " + str(amp_dtype)[6:]
+    print("%-5s %s batch=%d seq=%d: %6.1f ms/iteration  %6.1f samples/s  peak %5.2f GiB"
+          % (level, mode, batch, seq, median * 1e3, batch / median, torch.cuda.max_memory_allocated() / 2 ** 30), flush=True)
 
 
 if __name__ == "__main__":
@@ -66,9 +67,11 @@ if __name__ == "__main__":
     parser.add_argument("--batch", type=int, default=16)
     parser.add_argument("--seq", type=int, default=512)
     parser.add_argument("--steps", type=int, default=8)
-    parser.add_argument("--amp", action="store_true")
+    parser.add_argument("--amp", action="store_true", help="float16 autocast")
+    parser.add_argument("--amp-bf16", action="store_true", help="bfloat16 autocast")
     parser.add_argument("--levels", nargs="+", default=["L0", "L1", "L1.2"])
     args = parser.parse_args()
     for level in args.levels:
-        run(level, args.batch, args.seq, args.amp, args.steps)
+        run(level, args.batch, args.seq, args.amp or args.amp_bf16, args.steps,
+            torch.bfloat16 if args.amp_bf16 else torch.float16)
         torch.cuda.empty_cache()

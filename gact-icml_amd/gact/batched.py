@@ -42,9 +42,9 @@ class BatchedPacked:
         off = int(table_host[i, 5])
         so = self.owner.stats_offsets[i] * 4
         dt = self.dtypes[i]
-        esz = 4 if dt == torch.float32 else 2
-        sc = self.scale[so:so + N * esz].view(dt).reshape(N, 1, 1)
-        mn = self.min[so:so + N * esz].view(dt).reshape(N, 1, 1)
+        sdt = torch.float32 if dt == torch.bfloat16 else dt      # bfloat16 tensors keep a float scale
+        sc = self.scale[so:so + N * sdt.itemsize].view(sdt).reshape(N, 1, 1)
+        mn = self.min[so:so + N * dt.itemsize].view(dt).reshape(N, 1, 1)
         return self.packed[off:off + nbytes].view(torch.int8), b, sc, mn
 
 

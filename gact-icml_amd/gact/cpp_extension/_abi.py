@@ -11,11 +11,11 @@ import torch  # imported first so that the library binds to the HIP runtime torc
 _LIB = None
 LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "lib", "libgact_hip.so")
 
-F32, F16 = 0, 1
+F32, F16, BF16 = 0, 1, 2
 NOISE_CONST, NOISE_INJECT, NOISE_REF, NOISE_FAST = 0, 1, 2, 3
 NOISE_MODES = {"deterministic": NOISE_CONST, "inject": NOISE_INJECT, "reference": NOISE_REF, "fast": NOISE_FAST}
 GROUP = 256
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class BatchEntry(ctypes.Structure):
@@ -84,7 +84,9 @@ def dtype_code(dtype):
         return F32
     if dtype == torch.float16:
         return F16
-    raise RuntimeError("gact: only float32 and float16 are supported, got %s" % dtype)
+    if dtype == torch.bfloat16:     # the fused and the batched entry points only
+        return BF16
+    raise RuntimeError("gact: only float32, float16 and bfloat16 are supported, got %s" % dtype)
 
 
 def stream_of(t):

@@ -56,7 +56,7 @@ def no_scheme_quantize_pack(input, q_bit, seed, *, noise=None, rng_stream=None):
     if not input.is_cuda:
         raise RuntimeError("data must be a CUDA tensor!")
     dtype = input.dtype
-    if dtype is not torch.float32 and dtype is not torch.float16:
+    if dtype is not torch.float32 and dtype is not torch.float16 and dtype is not torch.bfloat16:
         raise RuntimeError("The type of data is not correct!")
     ext_quantization._check_bits(q_bit)
     seed = ext_quantization._seed_u64(seed)
@@ -76,9 +76,10 @@ def no_scheme_quantize_pack(input, q_bit, seed, *, noise=None, rng_stream=None):
                 raise RuntimeError("noise must be a contiguous float32 CUDA tensor with one value per padded element")
     device = x.device
     q_input = torch.empty(ext_quantization.packed_numel(q_bit, N, 1, _abi.GROUP), dtype=torch.int8, device=device)
-    q_scale = torch.empty((N, 1, 1), dtype=dtype, device=device)
+    # bfloat16 (not in the reference) is quantized as the float values it holds: float scale, bfloat16 min
+    q_scale = torch.empty((N, 1, 1), dtype=torch.float32 if dtype is torch.bfloat16 else dtype, device=device)
     q_min = torch.empty((N, 1, 1), dtype=dtype, device=device)
-    _abi.call_on(device, _abi.lib().gact_quantize, x.data_ptr(), _abi.F32 if dtype is torch.float32 else _abi.F16,
+    _abi.call_on(device, _abi.lib().gact_quantize, x.data_ptr(), _abi.dtype_code(dtype),
                  x.numel(), q_bit, mode, seed, None if noise is None else noise.data_ptr(), q_input.data_ptr(),
                  q_scale.data_ptr(), q_min.data_ptr(), None, torch._C._cuda_getCurrentRawStream(device.index))
     return q_input, q_scale, q_min
@@ -139,8 +140,8 @@ def op_dequantize(input, input_shape):
     if q_input.numel() < ext_quantization.packed_numel(q_bit, N, 1, _abi.GROUP) - 1 \
             or q_scale.numel() < N or q_min.numel() < N:
         raise RuntimeError("packed data / scale / min are too short for shape %s" % (tuple(input_shape),))
-    dtype = q_scale.dtype
-    if dtype is not q_min.dtype:
+    dtype = q_min.dtype      # the scale's type as well, except for bfloat16 tensors, whose scale is float
+    if q_scale.dtype is not (torch.float32 if dtype is torch.bfloat16 else dtype):
         raise RuntimeError("expected scalar type of min to match scale")
     device = q_input.device
     out = torch.empty(tuple(input_shape), dtype=dtype, device=device)

@@ -10,7 +10,7 @@ from .conf import config
 from .ops import op_dequantize, op_dequantize_mask, op_quantize, op_quantize_mask
 from .utils import sampled_key_with_sum
 
-_COMPRESSIBLE = (torch.float32, torch.float16)
+_COMPRESSIBLE = (torch.float32, torch.float16, torch.bfloat16)   # bfloat16: not in the reference
 _RANKS = (2, 3, 4)
 KEY_SAMPLES = 100
 BOOL_MASK_MIN_ELEMENTS = 4096     # smaller bool tensors are not worth a kernel launch
@@ -72,7 +72,7 @@ class Quantizer:
     def check_quantize(self, input_tensor):
         """-> (compress?, is it a 0/1 mask?).  The rules of quantizer.py:47-69 in their order: parameters stay;
         a non-empty uint8 tensor is a mask if it holds exactly the values 0 and 1 and is left alone otherwise;
-        then float16/float32 only, requires_grad only (batch-norm statistics do not), rank 2 to 4 only.
+        then float16 / float32 (and bfloat16, which the reference does not know) only, requires_grad only (batch-norm statistics do not), rank 2 to 4 only.
         One rule more than the reference has: a bool tensor on the GPU is a mask by construction (no
         values to inspect, no synchronisation) when config.compress_bool_masks is set."""
         t = input_tensor

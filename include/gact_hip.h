@@ -17,11 +17,16 @@
 extern "C" {
 #endif
 
-#define GACT_ABI_VERSION 2
+#define GACT_ABI_VERSION 3
 
 /* element types of activations, min, max and scale */
 #define GACT_F32 0
 #define GACT_F16 1
+/* bfloat16 activations (no counterpart in the reference, which knows float and half).  Taken by
+ * gact_quantize, gact_dequantize and the batched launches only.  min and max are bfloat16, the scale is
+ * FLOAT32: the codes, the scale and the minimum are those of the float path on the widened values, and
+ * dequantize rounds float(code) / scale + min to bfloat16, to nearest even. */
+#define GACT_BF16 2
 
 /* where the stochastic-rounding uniform u of each element comes from */
 #define GACT_NOISE_CONST 0  /* u = 0.5: deterministic round-to-nearest                          */
@@ -66,7 +71,7 @@ int gact_unpack(const void* packed, int bits, const void* scale, const void* mn,
 /* The whole of no_scheme_quantize_pack (gact/gact/ops.py:11-32) for group size 256 in one pass over
  * the data: `x` holds `numel` contiguous elements, treated as zero-padded to N = ceil(numel/256)
  * groups; writes min[N], scale[N] (and max[N] when `mx` is not null) and gact_packed_bytes(bits,N,1,256)
- * bytes.  Same results as gact_minimax + gact_pack on the padded tensor. */
+ * bytes.  Same results as gact_minimax + gact_pack on the padded tensor.  (GACT_BF16: scale is float32.) */
 int gact_quantize(const void* x, int dtype, int64_t numel, int bits, int noise_mode, uint64_t seed,
                   const float* noise, void* packed, void* scale, void* mn, void* mx, void* stream);
 
@@ -95,7 +100,7 @@ int gact_calc_precision_device(int32_t* b, const float* C, const int64_t* w, int
 typedef struct gact_batch_entry {
   const void* x;      /* activation (quantize input / dequantize output), numel elements          */
   int64_t numel;
-  int32_t dtype;      /* GACT_F32 / GACT_F16                                                       */
+  int32_t dtype;      /* GACT_F32 / GACT_F16 / GACT_BF16                                           */
   int32_t reserved;
   uint64_t seed;      /* per-tensor seed: seeds[tid] + seed_iter (gact/gact/quantizer.py:119-124)  */
   int64_t first_block; /* exclusive prefix sum of ceil(N/128) over the table (128 groups per block) */
@@ -119,12 +124,13 @@ int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int
  * tensor of every block; without it each block searches the table.  Results equal a loop of
  * gact_quantize / gact_dequantize over the tensors (gact/gact/quantizer.py:95-142 drives the reference
  * one tensor at a time).  `plan` is the array gact_batch_plan filled.  `dtypes` says which element types
- * occur in the table, which the host that built it knows: bit 0 float, bit 1 half (GACT_DTYPES_*); quantize
+ * occur in the table, which the host that built it knows: bit 0 float, bit 1 half, bit 2 bfloat16 (GACT_DTYPES_*); quantize
  * launches only the kernels of those types (a half-only kernel needs a third fewer registers than one that
  * also carries the float path), so a tensor whose type is missing from the mask is left unquantized. */
 #define GACT_DTYPES_F32 1
 #define GACT_DTYPES_F16 2
-#define GACT_DTYPES_ALL 3
+#define GACT_DTYPES_BF16 4
+#define GACT_DTYPES_ALL 7
 int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
                           int noise_mode, int dtypes, const int64_t* plan, const int32_t* block_map,
                           void* packed_arena, void* scale_arena, void* min_arena, void* stream);

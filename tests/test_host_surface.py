@@ -42,7 +42,7 @@ def test_struct_layout_matches_the_header():
 
 def test_status_codes_and_sizes():
     L = _abi.lib()
-    assert L.gact_abi_version() == 2
+    assert L.gact_abi_version() == 3
     assert L.gact_strerror(0) == b"ok"
     for code in (-1, -2, -3, -4, -5):
         assert L.gact_strerror(code) not in (b"ok", b"unknown error")
@@ -70,7 +70,10 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     assert L.gact_mask_pack(None, -1, None, None) == -1
     assert L.gact_calc_precision_device(16, 16, 16, 5000, 1.0, None, None) == -3                 # beyond the LDS table
     assert L.gact_quantize_batched(16, 16, 3, 3, 1, 3, 16, None, 16, 16, 16, None) == -1         # injected noise
-    assert L.gact_quantize_batched(16, 16, 3, 3, 0, 4, 16, None, 16, 16, 16, None) == -1         # dtype mask
+    assert L.gact_quantize_batched(16, 16, 3, 3, 0, 8, 16, None, 16, 16, 16, None) == -1         # dtype mask
+    assert L.gact_quantize(16, 3, 256, 4, 0, 0, None, 16, 16, 16, None, None) == -1               # element type
+    assert L.gact_quantize(0, 2, 256, 4, 0, 0, None, 16, 16, 16, None, None) == -1                # bfloat16, null data
+    assert L.gact_minimax(16, 2, 4, 64, 16, 16, None) == -1                                      # no bfloat16 here
 
 
 def test_python_faces_raise_the_reference_errors():
