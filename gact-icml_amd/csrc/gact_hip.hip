@@ -382,27 +382,32 @@ template <> struct Elem<bf16> {
   typedef float Stat;
   __device__ static __forceinline__ float stat_of(bf16 x) { return (float)x; }
   __device__ static __forceinline__ bf16 elem_of(float x) { return (bf16)x; }
-  struct Store { float v[2][8]; };
+  // the group stays in registers as loaded (pairs of bfloat16) and is widened where it is used - once for
+  // min / max, once for the codes: half the registers of a widened copy (1 bit: 8 groups per lane)
+  struct Store { uint32_t w[2][4]; };
+  __device__ static __forceinline__ float widen(const Store& st, int k, int e) {
+    const uint32_t w = st.w[k][e >> 1];
+    return __builtin_bit_cast(float, (e & 1) ? (w & 0xffff0000u) : (w << 16));
+  }
   __device__ static __forceinline__ void store_codes(uint8_t* p, const uint32_t (&b)[8]) { Elem<f16>::store_codes(p, b); }
   __device__ static __forceinline__ void load_noise(const float* p, float (&u)[8]) { Elem<f16>::load_noise(p, u); }
   __device__ static __forceinline__ void load_chunk(const bf16* p, Store& st, int k) {
     const u32x4 a = stream_load(reinterpret_cast<const u32x4*>(p));
-    const uint32_t w[4] = {a.x, a.y, a.z, a.w};
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      st.v[k][2 * j] = __builtin_bit_cast(float, w[j] << 16);
-      st.v[k][2 * j + 1] = __builtin_bit_cast(float, w[j] & 0xffff0000u);
-    }
+    st.w[k][0] = a.x; st.w[k][1] = a.y; st.w[k][2] = a.z; st.w[k][3] = a.w;
   }
-  __device__ static __forceinline__ void set(Store& st, int k, int e, bf16 x) { st.v[k][e] = (float)x; }
+  __device__ static __forceinline__ void set(Store& st, int k, int e, bf16 x) {
+    const uint32_t h = (uint32_t)__builtin_bit_cast(uint16_t, x);
+    if (e & 1) st.w[k][e >> 1] |= h << 16;   // the callers set a chunk's elements in order: the even one starts the pair
+    else st.w[k][e >> 1] = h;
+  }
   __device__ static __forceinline__ void group_minmax(const Store& st, float& lo_out, float& hi_out) {
     float lo = Elem<float>::init_lo(), hi = Elem<float>::init_hi();
 #pragma unroll
     for (int k = 0; k < 2; k++)
 #pragma unroll
       for (int e = 0; e < 8; e++) {
-        lo = __builtin_fminf(lo, st.v[k][e]);
-        hi = __builtin_fmaxf(hi, st.v[k][e]);
+        lo = __builtin_fminf(lo, widen(st, k, e));
+        hi = __builtin_fmaxf(hi, widen(st, k, e));
       }
     row_all_minmax(lo, hi);
     lo_out = lo;
@@ -412,7 +417,7 @@ template <> struct Elem<bf16> {
     return Elem<float>::make_scale(lo, hi, qmax);
   }
   __device__ static __forceinline__ uint32_t code1(const Store& st, int k, int e, float mn, float s, float u) {
-    float t = st.v[k][e] - mn;
+    float t = widen(st, k, e) - mn;
     float y = __builtin_fmaf(t, s, u);
     return rint_clamp0(y - 0.5f);
   }
