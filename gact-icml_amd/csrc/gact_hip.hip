@@ -1601,7 +1601,10 @@ inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8
 // lose, and keep full occupancy.
 // From 50 M elements on: with buffers that are cold in every cache the cap costs 3-12 % at 8-17 M elements,
 // is neutral at 34 M and gains 2-7 % at 50 M, 3-13 % at 84 M.
-constexpr int64_t kCapFromGroups = 3 << 16;
+#ifndef GACT_CAP_FROM_GROUPS
+#define GACT_CAP_FROM_GROUPS (3 << 16)
+#endif
+constexpr int64_t kCapFromGroups = GACT_CAP_FROM_GROUPS;
 inline unsigned dequantize_lds_cap(size_t elem_size, int bits, int64_t N) {
   if (N < kCapFromGroups) return 0u;
   if (elem_size == 4) return 53000u;
