@@ -12,8 +12,11 @@
 //
 // Dequantize has no reduction, so a unit of 8 consecutive groups goes to a whole wave (float: lane l owns
 // columns 4l .. 4l+3) or half a wave (half: 8l .. 8l+7): one 16-byte store per lane and group, every store
-// instruction writing whole groups contiguously.  At 1, 2 and 4 bit the 2^bits possible values of a group
-// are tabulated once in the lanes of a row and fetched with ds_bpermute.
+// instruction writing whole groups contiguously.  At 1, 2 and 4 bit the 8 * 2^bits possible values of a unit
+// are tabulated once across its lanes and fetched with ds_bpermute.
+//
+// Element types: float and half as in the reference; bfloat16 (an addition) is quantized as the float
+// values it holds, in the half layout.
 //
 // Workgroups are dealt to the 8 XCDs round-robin; xcd_tile() reorders the tiles so that each XCD's L2
 // streams runs of consecutive tiles.
@@ -148,7 +151,8 @@ __device__ __forceinline__ bool reciprocal_safe(float s) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Per-type pieces.  Store holds the 16 elements of one group a quantize lane owns (2 chunks of 8).
+// Per-type pieces.  Store holds the 16 elements of one group a quantize lane owns (float: 4 chunks of 4,
+// half and bfloat16: 2 chunks of 8).
 // ------------------------------------------------------------------------------------------------
 template <typename T> struct Elem;
 
