@@ -49,6 +49,8 @@ WORKLOADS = {
     "config3-gelu": ((16384, 4096), "float16", 4, "fast", "randn", "BERT-large GELU inputs fp16, 4 bit"),
     "config3-probs": ((32, 16, 512, 512), "float16", 2, "fast", "softmax", "BERT-large attention probs fp16, 2 bit"),
     "config4": ((169343, 256), "float32", 1, "fast", "relu60", "GCN node features fp32 [169343,256], ~60% zeros, 1 bit"),
+    # not a BASELINE workload: the GELU-input tensor of config 3 as mixed-precision training on this GPU holds it
+    "bf16-gelu": ((16384, 4096), "bfloat16", 4, "fast", "randn", "GELU inputs in bfloat16, 4 bit (float scale, bfloat16 min)"),
 }
 
 
@@ -64,11 +66,11 @@ def make_input(torch, shape, dtype, kind, seed=0):
     return x.to(getattr(torch, dtype)).contiguous()
 
 
-def algorithmic_bytes(numel, esize, bits):
+def algorithmic_bytes(numel, esize, bits, scale_esize=None):
     N = (numel + 255) // 256
     wpt = 8 // bits
     n_round = (N + wpt - 1) // wpt * wpt
-    return numel * esize + n_round * 32 * bits + 2 * N * esize
+    return numel * esize + n_round * 32 * bits + N * (esize + (scale_esize or esize))
 
 
 def run_workload(torch, name, steps, warmup, seed=42):
@@ -86,11 +88,12 @@ def run_workload(torch, name, steps, warmup, seed=42):
     packed_len = lib.gact_packed_bytes(bits, N, 1, 256) + 1
     working_set = 2 * numel * esize + packed_len
     sets = max(1, -(-ROTATE_BYTES // working_set))
+    scale_dtype = torch.float32 if x.dtype == torch.bfloat16 else x.dtype      # bfloat16 tensors keep a float scale
     bufs = []
     for r in range(sets):
         bufs.append((x if r == 0 else x.clone(),
                      torch.empty((packed_len,), dtype=torch.int8, device="cuda"),
-                     torch.empty((N,), dtype=x.dtype, device="cuda"), torch.empty((N,), dtype=x.dtype, device="cuda"),
+                     torch.empty((N,), dtype=scale_dtype, device="cuda"), torch.empty((N,), dtype=x.dtype, device="cuda"),
                      torch.empty_like(x)))
     st = torch.cuda.current_stream().cuda_stream
     dt = _abi.dtype_code(x.dtype)
@@ -133,7 +136,7 @@ def run_workload(torch, name, steps, warmup, seed=42):
         ev[k][2].record()
     torch.cuda.synchronize()
 
-    per_dir = algorithmic_bytes(numel, esize, bits)
+    per_dir = algorithmic_bytes(numel, esize, bits, 4 if x.dtype == torch.bfloat16 else None)
     q_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / steps
     d_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / steps
     res = {
@@ -331,7 +334,7 @@ def main():
         "metric": "quantize+dequantize GB/s (algorithmic input+output bytes), 1xMI355X, group=256",
         "value": res["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if res["dtype"] == "float32" else "f16", "data": "synthetic",
+        "dtype": {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[res["dtype"]], "data": "synthetic",
         "config": {"workload": "%s: %s" % (args.workload, res["desc"]), "bits": res["bits"], "group_size": 256,
                    "rng_stream": res["rng_stream"], "bytes_per_step": 2 * res["bytes_per_direction"]},
         "frac_of_hbm_peak": res["gbs"] / HBM_PEAK_GBS,
