@@ -66,6 +66,27 @@ __device__ __forceinline__ void row_all_minmax(float& lo, float& hi) {
 __device__ __forceinline__ void row_all_minmax(f16& lo, f16& hi) {
   asm(GACT_DPP_ALL("v_min_f16_dpp", "v_max_f16_dpp") : "+v"(lo), "+v"(hi));
 }
+// min / max across the 2 or 4 rows of a group of LANES lanes (32 or 64), after the row reduction: exchanges
+// with the lane 16 (and 32) away; every lane of the group ends with the result
+__device__ __forceinline__ float lane_xor(float v, int m) { return __shfl_xor(v, m, 64); }
+__device__ __forceinline__ f16 lane_xor(f16 v, int m) {
+  return __builtin_bit_cast(f16, (uint16_t)__shfl_xor((int)__builtin_bit_cast(uint16_t, v), m, 64));
+}
+__device__ __forceinline__ float min_of(float a, float b) { return __builtin_fminf(a, b); }
+__device__ __forceinline__ float max_of(float a, float b) { return __builtin_fmaxf(a, b); }
+__device__ __forceinline__ f16 min_of(f16 a, f16 b) { return __builtin_fminf16(a, b); }
+__device__ __forceinline__ f16 max_of(f16 a, f16 b) { return __builtin_fmaxf16(a, b); }
+template <int LANES, typename S>
+__device__ __forceinline__ void rows_all_minmax(S& lo, S& hi) {
+  if (LANES >= 32) {
+    lo = min_of(lo, lane_xor(lo, 16));
+    hi = max_of(hi, lane_xor(hi, 16));
+  }
+  if (LANES >= 64) {
+    lo = min_of(lo, lane_xor(lo, 32));
+    hi = max_of(hi, lane_xor(hi, 32));
+  }
+}
 
 // ------------------------------------------------------------------------------------------------
 // Philox4x32-10.  The key schedule only depends on the seed, so it stays on the scalar unit; each
@@ -174,20 +195,20 @@ template <> struct Elem<float> {
   __device__ static __forceinline__ float init_lo() { return 1e30f; }
   __device__ static __forceinline__ float init_hi() { return -1e30f; }
   __device__ static __forceinline__ float from_float(float v) { return v; }
-  __device__ static __forceinline__ void minmax(const Store& st, float& lo, float& hi) {
+  // min and max of the whole group, in every lane of the row
+  // CHN: chunks of the Store in use; LANES: lanes that share the group (16, or 32 / 64 with one chunk per lane)
+  template <int CHN = 4, int LANES = 16>
+  __device__ static __forceinline__ void group_minmax(const Store& st, float& lo_out, float& hi_out) {
+    float lo = init_lo(), hi = init_hi();
 #pragma unroll
-    for (int k = 0; k < 4; k++)
+    for (int k = 0; k < CHN; k++)
 #pragma unroll
       for (int e = 0; e < 4; e++) {
         lo = __builtin_fminf(lo, st.v[k][e]);
         hi = __builtin_fmaxf(hi, st.v[k][e]);
       }
-  }
-  // min and max of the whole group, in every lane of the row
-  __device__ static __forceinline__ void group_minmax(const Store& st, float& lo_out, float& hi_out) {
-    float lo = init_lo(), hi = init_hi();
-    minmax(st, lo, hi);
     row_all_minmax(lo, hi);
+    rows_all_minmax<LANES>(lo, hi);
     lo_out = lo;
     hi_out = hi;
   }
@@ -285,11 +306,12 @@ template <> struct Elem<f16> {
   // min and max of the whole group, in every lane of the row: packed per-lane min / max from +-inf (the
   // start values only survive in a lane whose 16 elements are all NaN), the two halves against each other,
   // then the row reduction
+  template <int CHN = 2, int LANES = 16>
   __device__ static __forceinline__ void group_minmax(const Store& st, f16& lo_out, f16& hi_out) {
     const f16 inf = (f16)__builtin_inff();
     f16x2 l = {inf, inf}, h = {(f16)-inf, (f16)-inf};
 #pragma unroll
-    for (int k = 0; k < 2; k++)
+    for (int k = 0; k < CHN; k++)
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         l = pk_min(l, st.v[k][j]);
@@ -301,6 +323,7 @@ template <> struct Elem<f16> {
     asm("v_max_f16_sdwa %0, %1, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1"
         : "=v"(hi) : "v"(h));
     row_all_minmax(lo, hi);
+    rows_all_minmax<LANES>(lo, hi);
     lo_out = lo;
     hi_out = hi;
   }
@@ -404,16 +427,18 @@ template <> struct Elem<bf16> {
     if (e & 1) st.w[k][e >> 1] |= h << 16;   // the callers set a chunk's elements in order: the even one starts the pair
     else st.w[k][e >> 1] = h;
   }
+  template <int CHN = 2, int LANES = 16>
   __device__ static __forceinline__ void group_minmax(const Store& st, float& lo_out, float& hi_out) {
     float lo = Elem<float>::init_lo(), hi = Elem<float>::init_hi();
 #pragma unroll
-    for (int k = 0; k < 2; k++)
+    for (int k = 0; k < CHN; k++)
 #pragma unroll
       for (int e = 0; e < 8; e++) {
         lo = __builtin_fminf(lo, widen(st, k, e));
         hi = __builtin_fmaxf(hi, widen(st, k, e));
       }
     row_all_minmax(lo, hi);
+    rows_all_minmax<LANES>(lo, hi);
     lo_out = lo;
     hi_out = hi;
   }
@@ -914,6 +939,178 @@ quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __re
   if (sg * (8 / BITS) >= N) return;
   quantize_supergroup<T, BITS, NOISE, GIVEN>(x, numel, N, sg, threadIdx.x & 15, packed, scale_out, mn_io, mx_io,
                                              (uint32_t)seed, (uint32_t)(seed >> 32), noise);
+}
+
+// The wide layout: one 16-byte chunk per lane and group, so GROUP / W lanes share a super-group - a whole wave
+// for float, half a wave for half and bfloat16 - and every load instruction reads whole groups.  With one
+// 16-lane row per super-group a wave of the float 1 bit kernel holds 32 KB in 128 registers per lane and the
+// kernel runs on few, long waves; here it holds 8 KB.  The row reductions are followed by one or two
+// exchanges across the rows; the byte of a column still belongs to one lane.  Same arithmetic (the same
+// Elem<T> functions on chunk 0 of a Store), same noise per element, same bytes.
+template <typename T, int BITS, int NOISE>
+__device__ __forceinline__ void quantize_supergroup_wide(const T* __restrict__ x, int64_t numel, int64_t N, int64_t sg,
+                                                         int l, uint8_t* __restrict__ packed,
+                                                         typename Elem<T>::Stat* __restrict__ scale_out,
+                                                         T* __restrict__ mn_out, T* __restrict__ mx_out, uint32_t k0,
+                                                         uint32_t k1, const float* __restrict__ noise) {
+  constexpr int WPT = 8 / BITS;
+  constexpr int QMAX = (1 << BITS) - 1;
+  constexpr int W = Elem<T>::kQWidth, LPS = GROUP / W;
+  static_assert(W == 8 || WPT >= 2, "4-column chunks pair two groups for the fast stream");
+  typedef typename Elem<T>::Stat Stat;
+  const int64_t n0 = sg * WPT;
+
+  typename Elem<T>::Store v[WPT];
+#pragma unroll
+  for (int ni = 0; ni < WPT; ni++) {
+    const int64_t n = n0 + ni;
+    if (n < N) {
+      const int64_t base = n * GROUP + W * l;
+      if (n * GROUP + GROUP <= numel) {
+        Elem<T>::load_chunk(x + base, v[ni], 0);
+      } else {
+#pragma unroll
+        for (int e = 0; e < W; e++) Elem<T>::set(v[ni], 0, e, base + e < numel ? x[base + e] : (T)0.0f);
+      }
+    }
+  }
+  Stat lo_t[WPT], hi_t[WPT], s_t[WPT];
+#pragma unroll
+  for (int ni = 0; ni < WPT; ni++) {
+    lo_t[ni] = (Stat)0.0f;
+    hi_t[ni] = (Stat)0.0f;
+    if (n0 + ni < N) Elem<T>::template group_minmax<1, LPS>(v[ni], lo_t[ni], hi_t[ni]);
+  }
+  // one scale division per lane: lane j of every row takes group j % WPT, then the row shares the results
+  {
+    const int mine = l & (WPT - 1);
+    Stat lo_m = lo_t[0], hi_m = hi_t[0];
+#pragma unroll
+    for (int ni = 1; ni < WPT; ni++) {
+      lo_m = (mine == ni) ? lo_t[ni] : lo_m;
+      hi_m = (mine == ni) ? hi_t[ni] : hi_m;
+    }
+    const Stat s_m = Elem<T>::make_scale(lo_m, hi_m, QMAX);
+    if (l < WPT && n0 + l < N) {
+      scale_out[n0 + l] = s_m;
+      mn_out[n0 + l] = Elem<T>::elem_of(lo_m);
+      if (mx_out) mx_out[n0 + l] = Elem<T>::elem_of(hi_m);
+    }
+    if (WPT == 1) {
+      s_t[0] = s_m;
+    } else {
+      s_t[0] = row_bcast<0>(s_m);
+      if (WPT > 1) s_t[1 % WPT] = row_bcast<1>(s_m);
+      if (WPT > 2) { s_t[2 % WPT] = row_bcast<2>(s_m); s_t[3 % WPT] = row_bcast<3>(s_m); }
+      if (WPT > 4) {
+        s_t[4 % WPT] = row_bcast<4>(s_m); s_t[5 % WPT] = row_bcast<5>(s_m);
+        s_t[6 % WPT] = row_bcast<6>(s_m); s_t[7 % WPT] = row_bcast<7>(s_m);
+      }
+    }
+  }
+
+  uint32_t bytes[W];
+#pragma unroll
+  for (int e = 0; e < W; e++) bytes[e] = 0;
+
+  if (NOISE == GACT_NOISE_REF) {
+#pragma unroll
+    for (int e = 0; e < W; e++) {
+      const uint64_t j = (uint64_t)sg * GROUP + W * l + e;
+      uint32_t r[4];
+#pragma unroll
+      for (int ni = 0; ni < WPT; ni++) {
+        if ((ni & 3) == 0) philox4x32_10(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r);
+        if (n0 + ni < N)
+          bytes[e] |= Elem<T>::code1(v[ni], 0, e, lo_t[ni], s_t[ni], curand_uniform_map(r[ni & 3])) << (ni * BITS);
+      }
+    }
+  } else {
+    constexpr int STEP = W == 8 ? 1 : 2;   // groups whose noise is drawn together
+#pragma unroll
+    for (int g = 0; g < WPT; g += STEP) {
+      float u[STEP][W];
+      if (NOISE == GACT_NOISE_FAST) {
+        if (W == 8) {
+          const uint64_t blk = (uint64_t)(n0 + g) * (GROUP / 8) + l;
+          uint32_t r[4];
+          philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
+#pragma unroll
+          for (int e = 0; e < W; e++) u[0][e] = fast_piece(r[(e >> 2) * 2], r[(e >> 2) * 2 + 1], e & 3);
+        } else {
+          // a Philox block feeds 8 consecutive elements = the columns of a pair of neighbouring lanes: the even
+          // lane computes the block of group g, the odd lane that of group g + 1, and they exchange halves
+          const bool odd = l & 1;
+          const uint64_t blk = (uint64_t)(n0 + g + (odd ? 1 : 0)) * (GROUP / 8) + (l >> 1);
+          uint32_t r[4];
+          philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
+          const uint32_t ga = swap_with_neighbour(odd ? r[0] : r[2]);
+          const uint32_t gb = swap_with_neighbour(odd ? r[1] : r[3]);
+          const uint32_t a0 = odd ? ga : r[0], a1 = odd ? gb : r[1];   // group g
+          const uint32_t b0 = odd ? r[2] : ga, b1 = odd ? r[3] : gb;   // group g + 1
+#pragma unroll
+          for (int e = 0; e < W; e++) {
+            u[0][e] = fast_piece(a0, a1, e);
+            u[STEP - 1][e] = fast_piece(b0, b1, e);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int h = 0; h < STEP; h++) {
+          if (NOISE == GACT_NOISE_INJECT && n0 + g + h < N) {
+            Elem<T>::load_noise(noise + (n0 + g + h) * GROUP + W * l, u[h]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < W; e++) u[h][e] = 0.5f;
+          }
+        }
+      }
+#pragma unroll
+      for (int h = 0; h < STEP; h++) {
+        const int ni = g + h;
+        if (n0 + ni < N) {
+          uint32_t c[W];
+          Elem<T>::template codes<NOISE == GACT_NOISE_CONST>(v[ni], 0, lo_t[ni], s_t[ni], u[h], c);
+#pragma unroll
+          for (int e = 0; e < W; e++) bytes[e] |= c[e] << (ni * BITS);
+        }
+      }
+    }
+  }
+  Elem<T>::store_codes(packed + sg * GROUP + W * l, bytes);
+}
+
+// Which (type, width) pairs take the wide layout in the single-tensor fused quantize, as bit sets of widths.
+// Measured on buffers that are cold in every cache (us, row layout -> wide layout): float 1 bit 35.4 -> 33.0 at
+// 43 M elements and 71.2 -> 68.7 at 103 M (no change at 17 / 50 / 134 M), bfloat16 1 bit 32.6 -> 30.6 at 50 M and
+// 75.9 -> 70.8 at 134 M.  Every other pair loses 2-30 % (half 1 bit 65.5 -> 69.5, float 4 bit 92.9 -> 106.4 at
+// 134 M): their rows already hold 8 KB per wave or less.
+#ifndef GACT_Q_WIDE_MASK_F32
+#define GACT_Q_WIDE_MASK_F32 0x1
+#endif
+#ifndef GACT_Q_WIDE_MASK_F16
+#define GACT_Q_WIDE_MASK_F16 0x0
+#endif
+#ifndef GACT_Q_WIDE_MASK_BF16
+#define GACT_Q_WIDE_MASK_BF16 0x1
+#endif
+template <typename T>
+__host__ __device__ constexpr bool quantize_is_wide(int bits) {
+  return ((Elem<T>::kDtype == GACT_F32 ? GACT_Q_WIDE_MASK_F32
+                                        : Elem<T>::kDtype == GACT_F16 ? GACT_Q_WIDE_MASK_F16 : GACT_Q_WIDE_MASK_BF16) &
+          bits) != 0;
+}
+
+template <typename T, int BITS, int NOISE>
+__global__ void __launch_bounds__(256)
+quantize_wide_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
+                     typename Elem<T>::Stat* __restrict__ scale_out, T* __restrict__ mn_out, T* __restrict__ mx_out,
+                     uint64_t seed, const float* __restrict__ noise) {
+  constexpr int LPS = GROUP / Elem<T>::kQWidth;
+  const int64_t sg = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / LPS;
+  if (sg * (8 / BITS) >= N) return;
+  quantize_supergroup_wide<T, BITS, NOISE>(x, numel, N, sg, threadIdx.x % LPS, packed, scale_out, mn_out, mx_out,
+                                           (uint32_t)seed, (uint32_t)(seed >> 32), noise);
 }
 
 template <typename T, int BITS>
@@ -1623,6 +1820,27 @@ template <typename T, int BITS, bool GIVEN>
 int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, typename Elem<T>::Stat* scale, T* mn, T* mx,
                     int noise_mode,
                     uint64_t seed, const float* noise, hipStream_t stream) {
+  if constexpr (!GIVEN && quantize_is_wide<T>(BITS) && (Elem<T>::kQWidth == 8 || BITS < 8)) {
+    const int64_t per_block = 256 / (GROUP / Elem<T>::kQWidth);
+    const dim3 wgrid((unsigned)((supergroups(N, BITS) + per_block - 1) / per_block)), wblock(256);
+    switch (noise_mode) {
+      case GACT_NOISE_CONST:
+        hipLaunchKernelGGL((quantize_wide_kernel<T, BITS, GACT_NOISE_CONST>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
+        break;
+      case GACT_NOISE_INJECT:
+        hipLaunchKernelGGL((quantize_wide_kernel<T, BITS, GACT_NOISE_INJECT>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
+        break;
+      case GACT_NOISE_REF:
+        hipLaunchKernelGGL((quantize_wide_kernel<T, BITS, GACT_NOISE_REF>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
+        break;
+      case GACT_NOISE_FAST:
+        hipLaunchKernelGGL((quantize_wide_kernel<T, BITS, GACT_NOISE_FAST>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
+        break;
+      default:
+        return GACT_EINVAL;
+    }
+    return launch_status();
+  }
   dim3 grid, block;
   row_grid(supergroups(N, BITS), &grid, &block, quantize_threads(BITS, sizeof(T)));
   // the reference stream's one Philox block per byte makes the kernel instruction-bound: it wants every wave
