@@ -1081,10 +1081,10 @@ __device__ __forceinline__ void quantize_supergroup_wide(const T* __restrict__ x
 }
 
 // Which (type, width) pairs take the wide layout in the single-tensor fused quantize, as bit sets of widths.
-// Measured on buffers that are cold in every cache (us, row layout -> wide layout): float 1 bit 35.4 -> 33.0 at
-// 43 M elements and 71.2 -> 68.7 at 103 M (no change at 17 / 50 / 134 M), bfloat16 1 bit 32.6 -> 30.6 at 50 M and
-// 75.9 -> 70.8 at 134 M.  Every other pair loses 2-30 % (half 1 bit 65.5 -> 69.5, float 4 bit 92.9 -> 106.4 at
-// 134 M): their rows already hold 8 KB per wave or less.
+// Measured on buffers that are cold in every cache (us, row layout -> wide layout): float 1 bit 36.5 -> 35.0 at
+// 43 M elements, even at 17 - 75 M, either sign from 103 M on (the launch keeps the row layout there);
+// bfloat16 1 bit 30.0 -> 27.3 at 43 M, 75.9 -> 70.8 at 134 M.  Every other pair loses 2-30 % (half 1 bit
+// 65.5 -> 69.5, float 4 bit 92.9 -> 106.4 at 134 M): their rows already hold 8 KB per wave or less.
 #ifndef GACT_Q_WIDE_MASK_F32
 #define GACT_Q_WIDE_MASK_F32 0x1
 #endif
@@ -1820,7 +1820,10 @@ template <typename T, int BITS, bool GIVEN>
 int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, typename Elem<T>::Stat* scale, T* mn, T* mx,
                     int noise_mode,
                     uint64_t seed, const float* noise, hipStream_t stream) {
-  if constexpr (!GIVEN && quantize_is_wide<T>(BITS) && (Elem<T>::kQWidth == 8 || BITS < 8)) {
+  // float: only below 50 M elements (43 M: 36.5 -> 35.0 us, 75 M: even, 103 M: 72.2 -> 73.8 us) - the shorter
+  // waves shorten the tail of a mid-sized launch, the long ones stream a little better once the tail is small
+  const bool wide_here = Elem<T>::kDtype != GACT_F32 || N < kCapFromGroups;
+  if constexpr (!GIVEN && quantize_is_wide<T>(BITS) && (Elem<T>::kQWidth == 8 || BITS < 8)) if (wide_here) {
     const int64_t per_block = 256 / (GROUP / Elem<T>::kQWidth);
     const dim3 wgrid((unsigned)((supergroups(N, BITS) + per_block - 1) / per_block)), wblock(256);
     switch (noise_mode) {
