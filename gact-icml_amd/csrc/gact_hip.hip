@@ -9,6 +9,8 @@
 // 8/bits consecutive groups into one byte - the lane that owns a column owns every code of that byte:
 // packing needs no cross-lane traffic at all.  One Philox block feeds 8 consecutive elements: a half
 // chunk, or the two float chunks of a pair of neighbouring lanes (which swap the halves they need).
+// Float and bfloat16 at 1 bit, whose rows would hold 8 groups in registers, spread a super-group over a
+// whole wave / half a wave instead (quantize_supergroup_wide): one chunk per lane and group.
 //
 // Dequantize has no reduction, so a unit of 8 consecutive groups goes to a whole wave (float: lane l owns
 // columns 4l .. 4l+3) or half a wave (half: 8l .. 8l+7): one 16-byte store per lane and group, every store
