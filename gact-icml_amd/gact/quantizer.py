@@ -83,7 +83,10 @@ class Quantizer:
             is_mask = (int(lo), int(hi)) == (0, 1)
             return is_mask, is_mask
         if t.dtype == torch.bool:
-            is_mask = config.compress_bool_masks and t.is_cuda and t.numel() >= BOOL_MASK_MIN_ELEMENTS
+            # contiguous only: an expanded or strided view (a broadcast attention mask) may occupy far less than
+            # numel bytes, and unpacking would hand back a dense copy
+            is_mask = (config.compress_bool_masks and t.is_cuda and t.numel() >= BOOL_MASK_MIN_ELEMENTS
+                       and t.is_contiguous())
             return is_mask, is_mask
         ok = t.dtype in _COMPRESSIBLE and t.requires_grad is not False and t.dim() in _RANKS
         return ok, False

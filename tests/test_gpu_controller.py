@@ -250,11 +250,14 @@ def test_saved_bool_masks_are_packed_to_one_bit_losslessly(monkeypatch):
     # the tuple protocol: a fourth entry carries the dtype; strided and small tensors
     q = quantizer_mod.Quantizer(default_bit=4, swap=False, prefetch=False)
     m = torch.rand(300, 130, device="cuda") < 0.5
-    for t in (m, m.t(), m[::2, 1::3].repeat(3, 5)):
+    for t in (m, m.t().contiguous(), m[::2, 1::3].repeat(3, 5), m.reshape(3, 100, 130)):
         h = q.quantize(t)
         assert h[:2] == (True, True) and h[3] == torch.bool
         back = q.dequantize(h)
         assert back.dtype == torch.bool and back.shape == t.shape and torch.equal(back, t)
+    # views that are not contiguous are left alone: a broadcast mask occupies less than it looks
+    for t in (m.t(), m[:1].expand(300, 130), m[::2]):
+        assert q.quantize(t)[0] is False
     small = torch.rand(10, 10, device="cuda") < 0.5
     assert q.quantize(small) == (False, small) or q.quantize(small)[1] is small
     config.compress_bool_masks = False
