@@ -74,10 +74,28 @@ __device__ __forceinline__ float lane_xor(float v, int m) { return __shfl_xor(v,
 __device__ __forceinline__ f16 lane_xor(f16 v, int m) {
   return __builtin_bit_cast(f16, (uint16_t)__shfl_xor((int)__builtin_bit_cast(uint16_t, v), m, 64));
 }
-__device__ __forceinline__ float min_of(float a, float b) { return __builtin_fminf(a, b); }
-__device__ __forceinline__ float max_of(float a, float b) { return __builtin_fmaxf(a, b); }
-__device__ __forceinline__ f16 min_of(f16 a, f16 b) { return __builtin_fminf16(a, b); }
-__device__ __forceinline__ f16 max_of(f16 a, f16 b) { return __builtin_fmaxf16(a, b); }
+// neither operand is NaN here (see row_all_minmax), so the bare instruction will do: the compiler's minnum /
+// maxnum put a canonicalising v_max v, v, v in front of every operand
+__device__ __forceinline__ float min_of(float a, float b) {
+  float r;
+  asm("v_min_f32_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ float max_of(float a, float b) {
+  float r;
+  asm("v_max_f32_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ f16 min_of(f16 a, f16 b) {
+  f16 r;
+  asm("v_min_f16_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ f16 max_of(f16 a, f16 b) {
+  f16 r;
+  asm("v_max_f16_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
 template <int LANES, typename S>
 __device__ __forceinline__ void rows_all_minmax(S& lo, S& hi) {
   if (LANES >= 32) {
