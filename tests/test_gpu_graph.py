@@ -34,3 +34,57 @@ def test_captured_pair_replays_like_eager(dtype, bits, stream):
         assert torch.equal(q[0][:-1], eq[0][:-1]), "replay %d: packed bytes" % rep
         assert torch.equal(q[2], eq[2]) and torch.equal(q[3], eq[3])
         assert torch.equal(out, eout), "replay %d: dequantized" % rep
+
+
+def test_whole_training_step_under_the_hooks_replays_as_a_graph():
+    """The hooks only allocate and launch (no synchronisation for float tensors), so a forward + backward pass
+    under them can be captured whole; replays on new data must give the gradients of the eager hooked step on
+    that data (the seeds are those of the captured iteration, which the eager step is given as well).  Several
+    replays with eager work and synchronisations in between, each one checked."""
+    import gact
+    from gact.conf import config
+    from gact.controller import Controller
+
+    saved = dict(vars(config))
+    try:
+        torch.manual_seed(0)
+        net = torch.nn.Sequential(torch.nn.Linear(512, 1024), torch.nn.GELU(), torch.nn.Linear(1024, 1024),
+                                  torch.nn.ReLU(), torch.nn.Linear(1024, 10)).cuda()
+        x = torch.randn(256, 512, device="cuda")
+        y = torch.randint(0, 10, (256,), device="cuda")
+        gact.set_optimization_level("L1")
+        ctl = Controller(net)
+        ctl.install_hook()
+        try:
+            def step():
+                net.zero_grad(set_to_none=False)
+                loss = torch.nn.functional.cross_entropy(net(x), y)
+                loss.backward()
+                ctl.quantizer.iterate()                     # tensor ids restart; the seed offset stays
+                return loss
+
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    step()
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                captured_loss = step()
+            assert len(ctl.quantizer.bits) >= 3
+            for trial in range(4):
+                x.copy_(torch.randn(256, 512, generator=torch.Generator().manual_seed(trial)).cuda())
+                graph.replay()
+                torch.cuda.synchronize()
+                got = torch.cat([p.grad.ravel() for p in net.parameters()]).clone()
+                got_loss = captured_loss.item()
+                eager_loss = step().item()
+                torch.cuda.synchronize()
+                want = torch.cat([p.grad.ravel() for p in net.parameters()])
+                assert got_loss == eager_loss, trial
+                assert torch.equal(got, want), (trial, (got - want).abs().max().item())
+        finally:
+            ctl.uninstall_hook()
+    finally:
+        vars(config).update(saved)
