@@ -15,6 +15,11 @@ from .cpp_extension import _abi
 from .cpp_extension import quantization as ext_quantization
 
 
+# the raw HIP stream torch currently launches on for a device (what _abi.stream_of wraps), bound once: these two
+# operators run once per saved tensor and iteration
+_current_stream = torch._C._cuda_getCurrentRawStream
+
+
 def _num_groups(numel):
     return (numel + config.group_size - 1) // config.group_size
 
@@ -81,7 +86,7 @@ def no_scheme_quantize_pack(input, q_bit, seed, *, noise=None, rng_stream=None):
     q_min = torch.empty((N, 1, 1), dtype=dtype, device=device)
     _abi.call_on(device, _abi.lib().gact_quantize, x.data_ptr(), _abi.dtype_code(dtype),
                  x.numel(), q_bit, mode, seed, None if noise is None else noise.data_ptr(), q_input.data_ptr(),
-                 q_scale.data_ptr(), q_min.data_ptr(), None, torch._C._cuda_getCurrentRawStream(device.index))
+                 q_scale.data_ptr(), q_min.data_ptr(), None, _current_stream(device.index))
     return q_input, q_scale, q_min
 
 
@@ -146,5 +151,5 @@ def op_dequantize(input, input_shape):
     device = q_input.device
     out = torch.empty(tuple(input_shape), dtype=dtype, device=device)
     _abi.call_on(device, _abi.lib().gact_dequantize, q_input.data_ptr(), q_bit, q_scale.data_ptr(), q_min.data_ptr(),
-                 _abi.dtype_code(dtype), num_features, out.data_ptr(), torch._C._cuda_getCurrentRawStream(device.index))
+                 _abi.dtype_code(dtype), num_features, out.data_ptr(), _current_stream(device.index))
     return out
