@@ -948,15 +948,25 @@ __device__ __forceinline__ uint32_t xcd_tile(uint32_t b, uint32_t nb) {
   return ((q / (RUN ? RUN : 1)) * XCDS + x) * (RUN ? RUN : 1) + q % (RUN ? RUN : 1);
 }
 
+// The seed of a launch: a host value plus, optionally, a value read from device memory when the kernel runs -
+// so that a launch recorded in a HIP graph draws fresh noise on every replay (the host updates the device word
+// between replays).
+struct SeedArg {
+  uint64_t seed;
+  const uint64_t* add;  // device pointer or null
+  __device__ __forceinline__ uint64_t value() const { return add ? seed + *add : seed; }
+};
+
 // One super-group per 16-lane row: short waves, many of them.
 template <typename T, int BITS, int NOISE, bool GIVEN>
 __global__ void __launch_bounds__(256)
 quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
-                typename Elem<T>::Stat* __restrict__ scale_out, T* mn_io, T* mx_io, uint64_t seed,
+                typename Elem<T>::Stat* __restrict__ scale_out, T* mn_io, T* mx_io, SeedArg seed_arg,
                 const float* __restrict__ noise) {
   constexpr uint32_t RUN = BITS >= 4 ? GACT_XCD_RUN_Q : GACT_XCD_RUN_Q_LOW;
   const int64_t sg = (int64_t)xcd_tile<RUN>(blockIdx.x, gridDim.x) * (blockDim.x >> 4) + (threadIdx.x >> 4);
   if (sg * (8 / BITS) >= N) return;
+  const uint64_t seed = seed_arg.value();
   quantize_supergroup<T, BITS, NOISE, GIVEN>(x, numel, N, sg, threadIdx.x & 15, packed, scale_out, mn_io, mx_io,
                                              (uint32_t)seed, (uint32_t)(seed >> 32), noise);
 }
@@ -1125,10 +1135,11 @@ template <typename T, int BITS, int NOISE>
 __global__ void __launch_bounds__(256)
 quantize_wide_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
                      typename Elem<T>::Stat* __restrict__ scale_out, T* __restrict__ mn_out, T* __restrict__ mx_out,
-                     uint64_t seed, const float* __restrict__ noise) {
+                     SeedArg seed_arg, const float* __restrict__ noise) {
   constexpr int LPS = GROUP / Elem<T>::kQWidth;
   const int64_t sg = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / LPS;
   if (sg * (8 / BITS) >= N) return;
+  const uint64_t seed = seed_arg.value();
   quantize_supergroup_wide<T, BITS, NOISE>(x, numel, N, sg, threadIdx.x % LPS, packed, scale_out, mn_out, mx_out,
                                            (uint32_t)seed, (uint32_t)(seed >> 32), noise);
 }
@@ -1839,7 +1850,7 @@ inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
 template <typename T, int BITS, bool GIVEN>
 int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, typename Elem<T>::Stat* scale, T* mn, T* mx,
                     int noise_mode,
-                    uint64_t seed, const float* noise, hipStream_t stream) {
+                    SeedArg seed, const float* noise, hipStream_t stream) {
   // float: only below 50 M elements (43 M: 36.5 -> 35.0 us, 75 M: even, 103 M: 72.2 -> 73.8 us) - the shorter
   // waves shorten the tail of a mid-sized launch, the long ones stream a little better once the tail is small
   const bool wide_here = Elem<T>::kDtype != GACT_F32 || N < kCapFromGroups;
@@ -1894,7 +1905,7 @@ int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, typen
 template <typename T, bool GIVEN>
 int dispatch_quantize(int bits, const T* x, int64_t numel, int64_t N, uint8_t* packed, typename Elem<T>::Stat* scale,
                       T* mn, T* mx,
-                      int noise_mode, uint64_t seed, const float* noise, hipStream_t stream) {
+                      int noise_mode, SeedArg seed, const float* noise, hipStream_t stream) {
   switch (bits) {
     case 1: return launch_quantize<T, 1, GIVEN>(x, numel, N, packed, scale, mn, mx, noise_mode, seed, noise, stream);
     case 2: return launch_quantize<T, 2, GIVEN>(x, numel, N, packed, scale, mn, mx, noise_mode, seed, noise, stream);
@@ -2057,9 +2068,9 @@ int gact_pack(const void* data, const void* mn, const void* mx, int dtype, int b
     // the fused row kernel with min/max taken from the caller
     if (dtype == GACT_F32)
       return dispatch_quantize<float, true>(bits, (const float*)data, N * GROUP, N, (uint8_t*)packed, (float*)scale,
-                                            (float*)const_cast<void*>(mn), (float*)const_cast<void*>(mx), noise_mode, seed, noise, s);
+                                            (float*)const_cast<void*>(mn), (float*)const_cast<void*>(mx), noise_mode, SeedArg{seed, nullptr}, noise, s);
     return dispatch_quantize<f16, true>(bits, (const f16*)data, N * GROUP, N, (uint8_t*)packed, (f16*)scale,
-                                        (f16*)const_cast<void*>(mn), (f16*)const_cast<void*>(mx), noise_mode, seed, noise, s);
+                                        (f16*)const_cast<void*>(mn), (f16*)const_cast<void*>(mx), noise_mode, SeedArg{seed, nullptr}, noise, s);
   }
   const int64_t count = N * G;
   const dim3 sgrid((unsigned)((count + 255) / 256)), sblock(256);
@@ -2089,8 +2100,9 @@ int gact_unpack(const void* packed, int bits, const void* scale, const void* mn,
   return unpack_any<f16>((const uint8_t*)packed, bits, (const f16*)scale, (const f16*)mn, N, G, D, (f16*)out, s);
 }
 
-int gact_quantize(const void* x, int dtype, int64_t numel, int bits, int noise_mode, uint64_t seed, const float* noise,
-                  void* packed, void* scale, void* mn, void* mx, void* stream) {
+int gact_quantize_seeded(const void* x, int dtype, int64_t numel, int bits, int noise_mode, uint64_t seed,
+                         const uint64_t* seed_add, const float* noise, void* packed, void* scale, void* mn, void* mx,
+                         void* stream) {
   if (dtype != GACT_F32 && dtype != GACT_F16 && dtype != GACT_BF16) return GACT_EINVAL;
   if (!valid_bits(bits) || numel < 0) return GACT_EINVAL;
   if (noise_mode < GACT_NOISE_CONST || noise_mode > GACT_NOISE_FAST) return GACT_EINVAL;
@@ -2098,13 +2110,20 @@ int gact_quantize(const void* x, int dtype, int64_t numel, int bits, int noise_m
   if (!x || !packed || !scale || !mn) return GACT_EINVAL;
   if (noise_mode == GACT_NOISE_INJECT && !noise) return GACT_EINVAL;
   if (!aligned16(x) || !aligned16(packed) || (noise_mode == GACT_NOISE_INJECT && !aligned16(noise))) return GACT_EALIGN;
+  if (reinterpret_cast<uintptr_t>(seed_add) & 7u) return GACT_EALIGN;
   const int64_t N = (numel + GROUP - 1) / GROUP;
   hipStream_t s = (hipStream_t)stream;
+  const SeedArg sa{seed, seed_add};
   if (dtype == GACT_F32)
-    return dispatch_quantize<float, false>(bits, (const float*)x, numel, N, (uint8_t*)packed, (float*)scale, (float*)mn, (float*)mx, noise_mode, seed, noise, s);
+    return dispatch_quantize<float, false>(bits, (const float*)x, numel, N, (uint8_t*)packed, (float*)scale, (float*)mn, (float*)mx, noise_mode, sa, noise, s);
   if (dtype == GACT_BF16)
-    return dispatch_quantize<bf16, false>(bits, (const bf16*)x, numel, N, (uint8_t*)packed, (float*)scale, (bf16*)mn, (bf16*)mx, noise_mode, seed, noise, s);
-  return dispatch_quantize<f16, false>(bits, (const f16*)x, numel, N, (uint8_t*)packed, (f16*)scale, (f16*)mn, (f16*)mx, noise_mode, seed, noise, s);
+    return dispatch_quantize<bf16, false>(bits, (const bf16*)x, numel, N, (uint8_t*)packed, (float*)scale, (bf16*)mn, (bf16*)mx, noise_mode, sa, noise, s);
+  return dispatch_quantize<f16, false>(bits, (const f16*)x, numel, N, (uint8_t*)packed, (f16*)scale, (f16*)mn, (f16*)mx, noise_mode, sa, noise, s);
+}
+
+int gact_quantize(const void* x, int dtype, int64_t numel, int bits, int noise_mode, uint64_t seed, const float* noise,
+                  void* packed, void* scale, void* mn, void* mx, void* stream) {
+  return gact_quantize_seeded(x, dtype, numel, bits, noise_mode, seed, nullptr, noise, packed, scale, mn, mx, stream);
 }
 
 int gact_dequantize(const void* packed, int bits, const void* scale, const void* mn, int dtype, int64_t numel, void* out,

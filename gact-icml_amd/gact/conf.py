@@ -34,6 +34,12 @@ class QuantizationConfig:
         # reference's uint8 rule never sees.  They are packed to one bit per element, losslessly.
         self.compress_bool_masks = True
 
+        # ---- seeds in device memory (not in the reference) ----
+        # The iteration count that is added to every tensor's seed is read by the kernels from a word in device
+        # memory instead of travelling as a launch argument.  Same noise; needed when the hooked pass is
+        # recorded in a HIP graph, whose launch arguments are frozen at capture.
+        self.device_seed = False
+
         # ---- stochastic-rounding noise (not in the reference) ----
         # "fast":          one Philox4x32-10 block per 8 elements, 16-bit uniforms
         # "reference":     the reference's stream (one Philox state per output byte, cuRAND uniform map)

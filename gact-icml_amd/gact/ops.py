@@ -39,8 +39,9 @@ def _padded_groups(input):
     return input.reshape(-1, group)
 
 
-def no_scheme_quantize_pack(input, q_bit, seed, *, noise=None, rng_stream=None):
-    """gact/gact/ops.py:11-32 -> (q_input, q_scale, q_min)."""
+def no_scheme_quantize_pack(input, q_bit, seed, *, noise=None, rng_stream=None, seed_offset=None):
+    """gact/gact/ops.py:11-32 -> (q_input, q_scale, q_min).  `seed_offset` (one int64 on the GPU, optional) is added
+    to `seed` when the kernel runs, for launches recorded in a HIP graph."""
     N = _num_groups(input.numel())
     if q_bit == 32:
         # the passthrough of ops.py:21-24: the padded [N, group] view itself, max - min, min
@@ -50,6 +51,8 @@ def no_scheme_quantize_pack(input, q_bit, seed, *, noise=None, rng_stream=None):
         return input_groups, q_scale, q_min
 
     if not _fused():
+        if seed_offset is not None:
+            raise RuntimeError("seed_offset needs the single-pass kernels (config.group_size 256)")
         from .cpp_extension import minimax as ext_minimax
         input_groups = _padded_groups(input.contiguous()).contiguous()
         q_min, mx = ext_minimax.minimax(input_groups)
@@ -84,9 +87,16 @@ def no_scheme_quantize_pack(input, q_bit, seed, *, noise=None, rng_stream=None):
     # bfloat16 (not in the reference) is quantized as the float values it holds: float scale, bfloat16 min
     q_scale = torch.empty((N, 1, 1), dtype=torch.float32 if dtype is torch.bfloat16 else dtype, device=device)
     q_min = torch.empty((N, 1, 1), dtype=dtype, device=device)
-    _abi.call_on(device, _abi.lib().gact_quantize, x.data_ptr(), _abi.dtype_code(dtype),
-                 x.numel(), q_bit, mode, seed, None if noise is None else noise.data_ptr(), q_input.data_ptr(),
-                 q_scale.data_ptr(), q_min.data_ptr(), None, _current_stream(device.index))
+    if seed_offset is None:
+        _abi.call_on(device, _abi.lib().gact_quantize, x.data_ptr(), _abi.dtype_code(dtype),
+                     x.numel(), q_bit, mode, seed, None if noise is None else noise.data_ptr(), q_input.data_ptr(),
+                     q_scale.data_ptr(), q_min.data_ptr(), None, _current_stream(device.index))
+    else:
+        if seed_offset.dtype is not torch.int64 or seed_offset.numel() != 1 or seed_offset.device != device:
+            raise RuntimeError("seed_offset must be one int64 on the device of the data")
+        _abi.call_on(device, _abi.lib().gact_quantize_seeded, x.data_ptr(), _abi.dtype_code(dtype),
+                     x.numel(), q_bit, mode, seed, seed_offset.data_ptr(), None if noise is None else noise.data_ptr(),
+                     q_input.data_ptr(), q_scale.data_ptr(), q_min.data_ptr(), None, _current_stream(device.index))
     return q_input, q_scale, q_min
 
 
@@ -116,9 +126,10 @@ def op_dequantize_mask(input):
     return output
 
 
-def op_quantize(input, q_bit, seed, *, noise=None, rng_stream=None):
+def op_quantize(input, q_bit, seed, *, noise=None, rng_stream=None, seed_offset=None):
     """gact/gact/ops.py:57-59 -> [q_input, q_bit, q_scale, q_min]."""
-    q_input, q_scale, q_min = no_scheme_quantize_pack(input, q_bit, seed, noise=noise, rng_stream=rng_stream)
+    q_input, q_scale, q_min = no_scheme_quantize_pack(input, q_bit, seed, noise=noise, rng_stream=rng_stream,
+                                                      seed_offset=seed_offset)
     return [q_input, q_bit, q_scale, q_min]
 
 

@@ -46,7 +46,18 @@ class Quantizer:
         # filled on the first iteration; read and rewritten by auto precision
         self.bits, self.dims, self.seeds = {}, {}, {}
         self.iter = 0        # iterations seen, the extra passes of auto precision included
+        self._seed_dev = None   # config.device_seed: seed_iter as one int64 on the GPU, created on first use
         self.seed_iter = 0   # added to every seed; constant during one adaptive step so that probes are comparable
+
+    @property
+    def seed_iter(self):
+        return self._seed_iter
+
+    @seed_iter.setter
+    def seed_iter(self, value):
+        self._seed_iter = value
+        if self._seed_dev is not None:
+            self._seed_dev.fill_(value)       # an eager fill between graph replays
 
     # ---- streams of the swap path under their reference names ----
     @property
@@ -128,7 +139,12 @@ class Quantizer:
     def _compress(self, t, tid):
         if self.iter == 0:      # the first pass fixes the tables auto precision works on
             self.bits[tid], self.dims[tid], self.seeds[tid] = self.default_bit, t.numel(), tid
-        q_inputs = op_quantize(t, self.bits[tid], self.seeds[tid] + self.seed_iter)
+        if config.device_seed:
+            if self._seed_dev is None:      # during the eager warm-up passes, never inside a capture
+                self._seed_dev = torch.full((1,), self._seed_iter, dtype=torch.int64, device=t.device)
+            q_inputs = op_quantize(t, self.bits[tid], self.seeds[tid], seed_offset=self._seed_dev)
+        else:
+            q_inputs = op_quantize(t, self.bits[tid], self.seeds[tid] + self.seed_iter)
         if self.swap:
             # On the current stream, as in the reference (quantizer.py:125-137, whose side-stream lines are
             # commented out).  Issuing the copy on the swap-out stream (wait_stream + record_stream) was

@@ -17,7 +17,7 @@
 extern "C" {
 #endif
 
-#define GACT_ABI_VERSION 3
+#define GACT_ABI_VERSION 4
 
 /* element types of activations, min, max and scale */
 #define GACT_F32 0
@@ -74,6 +74,15 @@ int gact_unpack(const void* packed, int bits, const void* scale, const void* mn,
  * bytes.  Same results as gact_minimax + gact_pack on the padded tensor.  (GACT_BF16: scale is float32.) */
 int gact_quantize(const void* x, int dtype, int64_t numel, int bits, int noise_mode, uint64_t seed,
                   const float* noise, void* packed, void* scale, void* mn, void* mx, void* stream);
+
+/* gact_quantize with a second part of the seed that is read from device memory when the kernel runs: the
+ * streams are seeded with seed + *seed_add (seed_add: one uint64 in device memory, 8-byte aligned; null = 0).
+ * For launches recorded in a HIP graph, whose host arguments are frozen at capture: the caller rewrites the
+ * device word between replays (gact/gact/quantizer.py:119-124 adds the iteration count to every tensor's seed)
+ * and every replay draws fresh noise.  No counterpart in the reference. */
+int gact_quantize_seeded(const void* x, int dtype, int64_t numel, int bits, int noise_mode, uint64_t seed,
+                         const uint64_t* seed_add, const float* noise, void* packed, void* scale, void* mn,
+                         void* mx, void* stream);
 
 /* The whole of dequantize_and_unpack + the slice of op_dequantize (gact/gact/ops.py:34-47,61-69) for
  * group size 256: writes exactly `numel` elements. */

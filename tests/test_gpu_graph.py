@@ -36,7 +36,8 @@ def test_captured_pair_replays_like_eager(dtype, bits, stream):
         assert torch.equal(out, eout), "replay %d: dequantized" % rep
 
 
-def test_whole_training_step_under_the_hooks_replays_as_a_graph():
+@pytest.mark.parametrize("device_seed", [False, True], ids=["host-seed", "device-seed"])
+def test_whole_training_step_under_the_hooks_replays_as_a_graph(device_seed):
     """The hooks only allocate and launch (no synchronisation for float tensors), so a forward + backward pass
     under them can be captured whole; replays on new data must give the gradients of the eager hooked step on
     that data (the seeds are those of the captured iteration, which the eager step is given as well).  Several
@@ -53,6 +54,7 @@ def test_whole_training_step_under_the_hooks_replays_as_a_graph():
         x = torch.randn(256, 512, device="cuda")
         y = torch.randint(0, 10, (256,), device="cuda")
         gact.set_optimization_level("L1")
+        config.device_seed = device_seed     # the iteration count of the seeds read from device memory by the kernels
         ctl = Controller(net)
         ctl.install_hook()
         try:
@@ -73,8 +75,11 @@ def test_whole_training_step_under_the_hooks_replays_as_a_graph():
             with torch.cuda.graph(graph):
                 captured_loss = step()
             assert len(ctl.quantizer.bits) >= 3
+            seen = []
             for trial in range(4):
-                x.copy_(torch.randn(256, 512, generator=torch.Generator().manual_seed(trial)).cuda())
+                x.copy_(torch.randn(256, 512, generator=torch.Generator().manual_seed(trial % 2)).cuda())
+                if device_seed:
+                    ctl.quantizer.seed_iter = 10 + trial      # what Controller.iterate does once per iteration
                 graph.replay()
                 torch.cuda.synchronize()
                 got = torch.cat([p.grad.ravel() for p in net.parameters()]).clone()
@@ -85,6 +90,10 @@ def test_whole_training_step_under_the_hooks_replays_as_a_graph():
                 # the same kernels on the same data: equal up to what the GEMM library may reorder between launches
                 assert abs(got_loss - eager_loss) <= 1e-6 * abs(eager_loss), trial
                 assert (got - want).norm().item() <= 1e-5 * want.norm().item(), trial
+                seen.append(got)
+            # trials 0 / 2 and 1 / 3 saw the same data: with the seed in device memory the replays drew fresh
+            # noise, with the seed frozen at capture they repeat themselves
+            assert torch.equal(seen[0], seen[2]) != device_seed and torch.equal(seen[1], seen[3]) != device_seed
         finally:
             ctl.uninstall_hook()
     finally:

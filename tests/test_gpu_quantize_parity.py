@@ -319,3 +319,16 @@ def test_other_group_sizes_take_the_extension_sequence(group, dtype):
                 np.testing.assert_array_equal(out.cpu().numpy().view(it), ref.view(it))
     finally:
         config.group_size = saved
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f16"])
+def test_seed_offset_in_device_memory_equals_the_sum_on_the_host(dtype):
+    x = torch.randn((50, 300), generator=torch.Generator().manual_seed(8)).to(dtype).cuda()
+    offset = torch.tensor([12345], dtype=torch.int64, device="cuda")
+    for bits in BITS:
+        for stream in ("fast", "reference"):
+            a = ops.op_quantize(x, bits, 7 + 12345, rng_stream=stream)
+            b = ops.op_quantize(x, bits, 7, rng_stream=stream, seed_offset=offset)
+            assert torch.equal(a[0][:-1], b[0][:-1]) and torch.equal(a[2], b[2]) and torch.equal(a[3], b[3])
+    with pytest.raises(RuntimeError):
+        ops.op_quantize(x, 4, 7, seed_offset=offset.int())

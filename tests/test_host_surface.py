@@ -42,7 +42,7 @@ def test_struct_layout_matches_the_header():
 
 def test_status_codes_and_sizes():
     L = _abi.lib()
-    assert L.gact_abi_version() == 3
+    assert L.gact_abi_version() == 4
     assert L.gact_strerror(0) == b"ok"
     for code in (-1, -2, -3, -4, -5):
         assert L.gact_strerror(code) not in (b"ok", b"unknown error")
@@ -62,6 +62,7 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     assert L.gact_quantize(None, 0, 256, 2, 0, 0, None, None, None, None, None, None) == -1      # null pointers
     assert L.gact_quantize(None, 0, 0, 2, 0, 0, None, None, None, None, None, None) == 0         # empty: nothing to do
     assert L.gact_quantize(8, 0, 256, 2, 0, 0, None, 16, 16, 16, None, None) == -2               # misaligned x
+    assert L.gact_quantize_seeded(16, 0, 256, 2, 0, 0, 4, None, 16, 16, 16, None, None) == -2   # misaligned seed word
     assert L.gact_dequantize(16, 5, 16, 16, 0, 256, 16, None) == -1
     assert L.gact_minimax(16, 0, 4, 48, 16, 16, None) == -3                                      # D % 32 != 0
     assert L.gact_minimax(16, 0, 4, 32, 16, 16, None) == -3                                      # D > 32
