@@ -1,17 +1,23 @@
 #!/usr/bin/env python3
 """Throughput of the saved-activation compression path on one MI355X.
 
-One step = one fused quantize (min/max + scale + stochastic rounding + pack) followed by one
-dequantize (unpack + affine) of one synthetic activation tensor, through the C ABI, with the input
-already resident in HBM.  The default workload is the headline one ("config2"): a ResNet-50 conv
-activation, fp32 NCHW [128,256,56,56], post-ReLU, group 256, 4 bit, stochastic rounding with Philox
-seed 42.  Bytes are the algorithmic input + output bytes of both directions:
-numel*sizeof(T) + packed bytes + 2*N*sizeof(T) per direction.
+One step = one fused quantize (min/max + scale + rounding + pack) followed by one dequantize (unpack +
+affine) of one synthetic activation tensor, through the C ABI, with the input already resident in HBM.
+The headline workload is the one the metric string names ("2-bit group=256"): BASELINE.json's first
+configuration, a float32 [4096,1024] tensor ~N(0,1) at 2 bit with deterministic rounding ("config1").
+Every other BASELINE configuration is measured in the same run and reported under "configs".
+Bytes are the algorithmic input + output bytes: numel*sizeof(T) + packed bytes + 2*N*sizeof(T) per direction.
 
-Prints ONE JSON line.  `value` and `ms_per_step` come from K steps launched back to back between two
-synchronisations.  `roofline` is for the slower of the two kernels, timed in a second pass over the same
-K steps with an event pair around every launch on the stream the kernels run on; `cpu_baseline` is the C
-restatement of the reference arithmetic (oracle/) run with OpenMP on the host cores over a bounded sample.
+Timing.  The K steps of a block are recorded once into a HIP graph (the launches go through the C ABI on
+the capturing stream) and the graph is replayed between two events on that stream; blocks are repeated
+until at least one second has been measured (the rule of the reference's tests/timeit_v2.py:246-257), the
+mean over all timed steps is reported.  A tensor whose buffers would fit the 256 MB last-level cache is
+given several buffer sets used in rotation, so that every step streams from and to HBM.  The duration of
+each kernel comes from the same construction with K launches of that kernel alone; `roofline` is the
+slower of the two kernels of the headline workload.  `cpu_baseline` is the C restatement of the reference
+arithmetic (oracle/) with OpenMP on the host cores.
+
+Prints ONE JSON line.
 """
 import argparse
 import json
@@ -25,19 +31,16 @@ for _p in (ROOT, os.path.join(ROOT, "gact-icml_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+MIN_SECONDS = 1.0      # every timed loop runs at least this long
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
-# a copy kernel of known size (profiles/config2_fp32_4bit_quantize_dequantize.txt: the copy kernel reads
-# FETCH_SIZE x 1.99988 and WRITE_SIZE x 1.00000 KiB); None for workloads without a counter run
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size
+# in the same runs (profiles/<workload>_*.txt name the runs and the factors); absent = no counter run
 TRAFFIC_BYTES = {
     ("config2", "quantize"): 466.5e6,    # 411.1 MB read + 55.4 MB written; algorithmic 465.6 MB
     ("config2", "dequantize"): 465.7e6,  # 54.7 MB read + 411.1 MB written; algorithmic 465.6 MB
 }
 
-# BASELINE.json's metric, verbatim.  Its text says 2 bit while the configuration it is quoted on (configs[1], the
-# default workload here) is 4 bit: the line carries the default workload as `value` and the same tensor at
-# 2 bit under `two_bit_same_tensor`.
-BASELINE_METRIC = "quantize+dequantize GB/s and % of HBM peak, 1\u00d7MI355X, 2-bit group=256"
+BASELINE_METRIC = "quantize+dequantize GB/s and % of HBM peak, 1×MI355X, 2-bit group=256"
 
 # a workload whose buffers are smaller than this is timed over several buffer sets in rotation
 ROTATE_BYTES = 800 * 1000 * 1000
@@ -45,11 +48,10 @@ ROTATE_BYTES = 800 * 1000 * 1000
 WORKLOADS = {
     # name: (shape, dtype, bits, rng_stream, data kind, description)
     "config1": ((4096, 1024), "float32", 2, "deterministic", "randn",
-                "fp32 [4096,1024] ~N(0,1), 2 bit, deterministic rounding"),
+                "fp32 [4096,1024] ~N(0,1) seed 0, 2 bit, deterministic rounding"),
     "config2": ((128, 256, 56, 56), "float32", 4, "fast", "relu",
                 "ResNet-50 conv activation fp32 [128,256,56,56] post-ReLU, 4 bit, stochastic rounding, Philox seed 42"),
-    "config2-2bit": ((128, 256, 56, 56), "float32", 2, "fast", "relu",
-                     "config2's tensor at 2 bit (the width BASELINE.json's metric string names)"),
+    "config2-2bit": ((128, 256, 56, 56), "float32", 2, "fast", "relu", "config2's tensor at 2 bit"),
     "config2-refstream": ((128, 256, 56, 56), "float32", 4, "reference", "relu",
                           "config2 with the reference's one-Philox-state-per-byte noise stream"),
     "config3-hidden": ((16384, 1024), "float16", 8, "fast", "randn", "BERT-large hidden states fp16, 8 bit"),
@@ -59,6 +61,8 @@ WORKLOADS = {
     # not a BASELINE workload: the GELU-input tensor of config 3 as mixed-precision training on this GPU holds it
     "bf16-gelu": ((16384, 4096), "bfloat16", 4, "fast", "randn", "GELU inputs in bfloat16, 4 bit (float scale, bfloat16 min)"),
 }
+# what a default run measures besides the headline workload (config5 is the batched one)
+BASELINE_SET = ["config1", "config2", "config2-2bit", "config3-hidden", "config3-gelu", "config3-probs", "config4"]
 
 
 def make_input(torch, shape, dtype, kind, seed=0):
@@ -80,10 +84,51 @@ def algorithmic_bytes(numel, esize, bits, scale_esize=None):
     return numel * esize + n_round * 32 * bits + N * (esize + (scale_esize or esize))
 
 
-def run_workload(torch, name, steps, warmup, seed=42):
-    """One step = quantize then dequantize of the workload's tensor.  A tensor whose buffers would fit the
-    256 MB last-level cache is given several buffer sets used in rotation, so that every step streams from
-    and to HBM as it does inside a training step."""
+class Timer:
+    """Mean duration of fn(k) over blocks of `steps` calls, at least MIN_SECONDS of them."""
+
+    def __init__(self, torch, steps, warmup, min_seconds, graph=True):
+        self.torch, self.steps, self.warmup, self.min_seconds, self.graph = torch, steps, warmup, min_seconds, graph
+
+    def __call__(self, fn):
+        torch = self.torch
+        for k in range(self.warmup):
+            fn(k)
+        torch.cuda.synchronize()
+        block = None
+        if self.graph:
+            # the block's launches, recorded once on a side stream (capture cannot run on the null stream)
+            block = torch.cuda.CUDAGraph()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                with torch.cuda.graph(block, stream=side):
+                    for k in range(self.steps):
+                        fn(k)
+            torch.cuda.current_stream().wait_stream(side)
+            block.replay()      # untimed: the first replay uploads the graph
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        total_ms, calls = 0.0, 0
+        t_begin = time.perf_counter()
+        while True:
+            e0.record()
+            if block is not None:
+                block.replay()
+            else:
+                for k in range(self.steps):
+                    fn(k)
+            e1.record()
+            e1.synchronize()
+            total_ms += e0.elapsed_time(e1)
+            calls += self.steps
+            if time.perf_counter() - t_begin >= self.min_seconds:
+                break
+        return total_ms / calls, calls
+
+
+def run_workload(torch, name, timer, seed=42, keep_input=False):
+    """One step = quantize then dequantize of the workload's tensor."""
     from gact.cpp_extension import _abi
 
     shape, dtype, bits, stream, kind, desc = WORKLOADS[name]
@@ -102,61 +147,74 @@ def run_workload(torch, name, steps, warmup, seed=42):
                      torch.empty((packed_len,), dtype=torch.int8, device="cuda"),
                      torch.empty((N,), dtype=scale_dtype, device="cuda"), torch.empty((N,), dtype=x.dtype, device="cuda"),
                      torch.empty_like(x)))
-    st = torch.cuda.current_stream().cuda_stream
     dt = _abi.dtype_code(x.dtype)
     mode = _abi.NOISE_MODES[stream]
 
     def quantize(k):
         xi, packed, scale, mn, _ = bufs[k % sets]
         _abi.check(lib.gact_quantize(xi.data_ptr(), dt, numel, bits, mode, seed, None, packed.data_ptr(),
-                                     scale.data_ptr(), mn.data_ptr(), None, st))
+                                     scale.data_ptr(), mn.data_ptr(), None, torch.cuda.current_stream().cuda_stream))
 
     def dequantize(k):
         _, packed, scale, mn, out = bufs[k % sets]
         _abi.check(lib.gact_dequantize(packed.data_ptr(), bits, scale.data_ptr(), mn.data_ptr(), dt, numel,
-                                       out.data_ptr(), st))
+                                       out.data_ptr(), torch.cuda.current_stream().cuda_stream))
 
-    for k in range(max(warmup, sets)):
+    def step(k):
         quantize(k)
         dequantize(k)
 
-    # the timed steps: nothing but the launches between the two synchronisations
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(steps):
-        quantize(k)
-        dequantize(k)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    wall_ms = (t1 - t0) * 1e3 / steps
-
-    # the same steps again with an event pair around every launch, for the duration of each kernel (an
-    # event between two launches drains the pipeline, about 5 us per step, so this pass is not the one the
-    # step time comes from)
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
-    torch.cuda.synchronize()
-    for k in range(steps):
-        ev[k][0].record()
-        quantize(k)
-        ev[k][1].record()
-        dequantize(k)
-        ev[k][2].record()
-    torch.cuda.synchronize()
+    for k in range(sets):   # every set holds valid codes before a dequantize-only loop reads them
+        step(k)
+    step_ms, timed_steps = timer(step)
+    q_ms, _ = timer(quantize)
+    d_ms, _ = timer(dequantize)
 
     per_dir = algorithmic_bytes(numel, esize, bits, 4 if x.dtype == torch.bfloat16 else None)
-    q_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / steps
-    d_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / steps
+    gbs = lambda ms: per_dir / (ms * 1e-3) / 1e9
     res = {
         "workload": name, "desc": desc, "shape": list(shape), "dtype": dtype, "bits": bits, "rng_stream": stream,
-        "bytes_per_direction": per_dir, "buffer_sets": sets, "ms_per_step": wall_ms,
-        "gbs": 2 * per_dir / (wall_ms * 1e-3) / 1e9,
-        "quantize": {"ms": q_ms, "gbs": per_dir / (q_ms * 1e-3) / 1e9},
-        "dequantize": {"ms": d_ms, "gbs": per_dir / (d_ms * 1e-3) / 1e9},
+        "bytes_per_direction": per_dir, "buffer_sets": sets, "ms_per_step": step_ms, "timed_steps": timed_steps,
+        "gbs": 2 * per_dir / (step_ms * 1e-3) / 1e9,
+        "quantize": {"ms": q_ms, "gbs": gbs(q_ms)},
+        "dequantize": {"ms": d_ms, "gbs": gbs(d_ms)},
     }
-    return res, x
+    return res, (x if keep_input else None)
 
 
-def run_config5(torch, steps, warmup, seed=42):
+def run_ceilings(torch, timer):
+    """What this GPU's memory system gives plain streams over config2's tensor (411 MB), in the same run: the
+    runtime's device-to-device copy, a fill, and a pure read (the library's row min/max, which reads the tensor
+    with the fused kernel's access pattern and writes 2 values per 256)."""
+    from gact.cpp_extension import _abi
+
+    lib = _abi.lib()
+    shape, dtype, _, _, kind, _ = WORKLOADS["config2"]
+    x = make_input(torch, shape, dtype, kind)
+    y = torch.empty_like(x)
+    nbytes = x.numel() * x.element_size()
+    N = x.numel() // 256
+    mn = torch.empty((N,), dtype=x.dtype, device="cuda")
+    mx = torch.empty((N,), dtype=x.dtype, device="cuda")
+
+    def copy(k):
+        y.copy_(x)
+
+    def fill(k):
+        y.fill_(1.0)
+
+    def read(k):
+        _abi.check(lib.gact_minimax(x.data_ptr(), _abi.F32, N, 256, mn.data_ptr(), mx.data_ptr(),
+                                    torch.cuda.current_stream().cuda_stream))
+
+    out = {"tensor": "config2's (%d bytes)" % nbytes}
+    for name, fn, moved in (("device_copy", copy, 2 * nbytes), ("fill", fill, nbytes), ("read_minimax", read, nbytes + 8 * N)):
+        ms, _ = timer(fn)
+        out[name] = {"us": ms * 1e3, "gbs": moved / (ms * 1e-3) / 1e9, "frac": moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    return out
+
+
+def run_config5(torch, timer, seed=42):
     """Workload "config5", the full adaptive step: 120 fp16 tensors with Swin-Tiny-like shapes, per-tensor
     sensitivities ~LogNormal(0,2), budget 2 bits per element.  One step = greedy calc_precision on the GPU
     (widths stay in device memory), offset planning, one batched mixed-width quantize and one batched
@@ -186,101 +244,55 @@ def run_config5(torch, steps, warmup, seed=42):
     packed = torch.empty((bq.arena_bytes_for_budget(target),), dtype=torch.uint8, device="cuda")
     sc = torch.empty((bq.total_groups * 4,), dtype=torch.uint8, device="cuda")
     mn = torch.empty((bq.total_groups * 4,), dtype=torch.uint8, device="cuda")
-    plan = torch.empty((6,), dtype=torch.int64, device="cuda")
-    st = torch.cuda.current_stream().cuda_stream
+    ws_q, ws_d = bq.new_workspace(), bq.new_workspace()
+    cur = lambda: torch.cuda.current_stream().cuda_stream
 
-    def allocate():
+    def allocate(k):
         bits.copy_(init)
         _abi.check(lib.gact_calc_precision_device(bits.data_ptr(), C.data_ptr(), w.data_ptr(), L, target,
-                                                  status.data_ptr(), st))
+                                                  status.data_ptr(), cur()))
 
-    def quantize():
-        _abi.check(lib.gact_batch_plan(table_q.data_ptr(), bits.data_ptr(), L, packed.numel(), plan.data_ptr(), st))
-        _abi.check(lib.gact_quantize_batched(table_q.data_ptr(), bits.data_ptr(), L, bq.total_blocks, _abi.NOISE_FAST,
-                                             bq.dtype_mask, plan.data_ptr(), bq.block_map.data_ptr(), packed.data_ptr(),
-                                             sc.data_ptr(), mn.data_ptr(), st))
+    def quantize(k):
+        bq.launch_quantize(table_q, bits, packed, sc, mn, ws_q, _abi.NOISE_FAST)
 
-    def dequantize():
-        _abi.check(lib.gact_batch_plan(table_d.data_ptr(), bits.data_ptr(), L, packed.numel(), plan.data_ptr(), st))
-        _abi.check(lib.gact_dequantize_batched(table_d.data_ptr(), bits.data_ptr(), L, bq.total_blocks,
-                                               plan.data_ptr(), bq.block_map.data_ptr(), packed.data_ptr(),
-                                               sc.data_ptr(), mn.data_ptr(), st))
+    def dequantize(k):
+        bq.launch_dequantize(table_d, bits, packed, sc, mn, ws_d)
 
-    for _ in range(warmup):
-        allocate(); quantize(); dequantize()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(steps):
-        allocate(); quantize(); dequantize()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    wall_ms = (t1 - t0) * 1e3 / steps
+    def step(k):
+        allocate(k)
+        quantize(k)
+        dequantize(k)
 
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
-    for k in range(steps):
-        ev[k][0].record(); allocate()
-        ev[k][1].record(); quantize()
-        ev[k][2].record(); dequantize()
-        ev[k][3].record()
+    step(0)
+    step_ms, timed_steps = timer(step)
+    a_ms, _ = timer(allocate)
+    q_ms, _ = timer(quantize)
+    d_ms, _ = timer(dequantize)
     torch.cuda.synchronize()
     host_bits = bits.cpu().tolist()
-    assert status.item() == 0 and plan.cpu().tolist()[1] == 1
+    assert status.item() == 0 and bq.plan_ok(ws_q) and bq.plan_ok(ws_d)
     per_dir = sum(algorithmic_bytes(x.numel(), 2, b) for x, b in zip(xs, host_bits))
-    a_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / steps
-    q_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / steps
-    d_ms = sum(e[2].elapsed_time(e[3]) for e in ev) / steps
-
-    # the same tensors and widths one call per tensor (what a hook-driven loop does), for comparison
-    singles = []
-    for x, o, b, sd in zip(xs, outs, host_bits, seeds):
-        N = (x.numel() + 255) // 256
-        singles.append((x, o, b, sd, torch.empty((lib.gact_packed_bytes(b, N, 1, 256) + 1,), dtype=torch.int8, device="cuda"),
-                        torch.empty((N,), dtype=x.dtype, device="cuda"), torch.empty((N,), dtype=x.dtype, device="cuda")))
-
-    def loop_q():
-        for x, o, b, sd, pk, s1, m1 in singles:
-            lib.gact_quantize(x.data_ptr(), 1, x.numel(), b, _abi.NOISE_FAST, sd, None, pk.data_ptr(), s1.data_ptr(),
-                              m1.data_ptr(), None, st)
-
-    def loop_d():
-        for x, o, b, sd, pk, s1, m1 in singles:
-            lib.gact_dequantize(pk.data_ptr(), b, s1.data_ptr(), m1.data_ptr(), 1, x.numel(), o.data_ptr(), st)
-
-    loop_ms = []
-    for fn in (loop_q, loop_d):
-        fn()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(5):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        loop_ms.append(e0.elapsed_time(e1) / 5)
     return {
         "workload": "config5", "desc": "120 fp16 Swin-Tiny-like tensors, widths by calc_precision on the GPU (budget "
                                        "2 bits/element), one batched mixed-width quantize + dequantize",
         "tensors": L, "elements": int(sum(x.numel() for x in xs)), "dtype": "float16", "rng_stream": "fast",
-        "width_histogram": {str(b): host_bits.count(b) for b in (1, 2, 4, 8)},
-        "bytes_per_direction": per_dir, "ms_per_step": wall_ms, "gbs": 2 * per_dir / (wall_ms * 1e-3) / 1e9,
+        "bits": "1/2/4/8 by calc_precision", "width_histogram": {str(b): host_bits.count(b) for b in (1, 2, 4, 8)},
+        "bytes_per_direction": per_dir, "buffer_sets": 1, "ms_per_step": step_ms, "timed_steps": timed_steps,
+        "gbs": 2 * per_dir / (step_ms * 1e-3) / 1e9,
         "calc_precision": {"ms": a_ms},
         "quantize": {"ms": q_ms, "gbs": per_dir / (q_ms * 1e-3) / 1e9},
         "dequantize": {"ms": d_ms, "gbs": per_dir / (d_ms * 1e-3) / 1e9},
-        "tensor_by_tensor": {"quantize_ms": loop_ms[0], "dequantize_ms": loop_ms[1],
-                             "quantize_gbs": per_dir / (loop_ms[0] * 1e-3) / 1e9,
-                             "dequantize_gbs": per_dir / (loop_ms[1] * 1e-3) / 1e9},
     }
 
 
-def cpu_baseline(torch, x, bits, stream, budget_s=12.0):
-    """The C restatement on the host cores over a leading slice of the same tensor."""
-    import numpy as np
-
+def cpu_baseline(torch, x, bits, stream, budget_s=10.0, max_elems=1 << 23):
+    """The C restatement on the host cores: the whole tensor when it has at most 8 M elements, else a leading
+    slice of that size."""
     import oracle
 
     mode = {"deterministic": oracle.NOISE_CONST, "reference": oracle.NOISE_REF, "fast": oracle.NOISE_FAST}[stream]
     flat = x.reshape(-1)
-    sample_elems = min(flat.numel(), 256 * 32768)  # 8M elements
+    sample_elems = min(flat.numel(), max_elems) // 256 * 256
     xs = flat[:sample_elems].cpu().numpy()
     N = sample_elems // 256
     groups = xs.reshape(N, 256)
@@ -290,7 +302,7 @@ def cpu_baseline(torch, x, bits, stream, budget_s=12.0):
         q = oracle.op_quantize(groups, bits, mode, 42)
         oracle.op_dequantize(q, groups.shape)
 
-    one_pass()  # warm-up (also builds / loads the library)
+    one_pass()  # warm-up (also loads the library)
     t0 = time.perf_counter()
     reps = 0
     while True:
@@ -300,20 +312,41 @@ def cpu_baseline(torch, x, bits, stream, budget_s=12.0):
             break
     dt = (time.perf_counter() - t0) / reps
     per_dir = algorithmic_bytes(sample_elems, esize, bits)
+    what = "the whole tensor" if sample_elems == flat.numel() else "a sample: the first %d of %d elements" % (sample_elems, flat.numel())
     return {
         "value": 2 * per_dir / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
-        "sample": "first %d of %d elements of the same tensor (%d groups), %d quantize+dequantize passes of the C "
-                  "restatement (oracle/gact_oracle.c, OpenMP) in %.1f s" % (sample_elems, flat.numel(), N, reps, dt * reps),
+        "sample": "%s (%d groups), %d quantize+dequantize passes of the C restatement (oracle/gact_oracle.c, "
+                  "OpenMP) in %.1f s" % (what, N, reps, dt * reps),
     }
+
+
+def compact(res):
+    """The per-configuration entry of the JSON line."""
+    out = {
+        "desc": res["desc"], "dtype": res["dtype"], "bits": res["bits"], "bytes_per_direction": res["bytes_per_direction"],
+        "buffer_sets": res["buffer_sets"],
+        "step": {"us": res["ms_per_step"] * 1e3, "gbs": res["gbs"], "frac": res["gbs"] / HBM_PEAK_GBS},
+    }
+    for k in ("quantize", "dequantize"):
+        out[k] = {"us": res[k]["ms"] * 1e3, "gbs": res[k]["gbs"], "frac": res[k]["gbs"] / HBM_PEAK_GBS}
+    for k in ("width_histogram", "tensors", "elements"):
+        if k in res:
+            out[k] = res[k]
+    if "calc_precision" in res:
+        out["calc_precision_us"] = res["calc_precision"]["ms"] * 1e3
+    return out
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS) + ["config5"])
-    ap.add_argument("--all", action="store_true", help="also time the other single-tensor workloads (extra key)")
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="config1", choices=sorted(WORKLOADS) + ["config5"],
+                    help="the workload `value`, `roofline` and `cpu_baseline` are about")
+    ap.add_argument("--only", action="store_true", help="measure the headline workload only (profiling runs)")
+    ap.add_argument("--min-seconds", type=float, default=MIN_SECONDS, help="minimum measured time of every loop")
+    ap.add_argument("--eager", action="store_true", help="launch every step from the host instead of replaying a graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed region also launch 20 plain device copies of the workload tensor, so "
@@ -328,13 +361,18 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     torch.cuda.set_device(0)
+    timer = Timer(torch, args.steps, args.warmup, args.min_seconds, graph=not args.eager)
 
-    if args.workload == "config5":
-        res, x = run_config5(torch, args.steps, args.warmup), None
-        res.update(bits="1/2/4/8 by calc_precision", dtype="float16")
-        args.copy_calibration, args.no_cpu = False, True     # no single tensor to copy or to hand to the CPU leg
-    else:
-        res, x = run_workload(torch, args.workload, args.steps, args.warmup)
+    def run(name, keep_input=False):
+        if name == "config5":
+            # the batched step is milliseconds long and allocates nothing: launched from the host
+            return run_config5(torch, Timer(torch, max(5, args.steps // 5), max(2, args.warmup // 5), args.min_seconds,
+                                            graph=False)), None
+        r = run_workload(torch, name, timer, keep_input=keep_input)
+        torch.cuda.empty_cache()
+        return r
+
+    res, x = run(args.workload, keep_input=True)
     dom = "quantize" if res["quantize"]["ms"] >= res["dequantize"]["ms"] else "dequantize"
     achieved = res[dom]["gbs"]
     line = {
@@ -343,20 +381,19 @@ def main():
         "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[res["dtype"]], "data": "synthetic",
         "config": {"workload": "%s: %s" % (args.workload, res["desc"]), "bits": res["bits"], "group_size": 256,
-                   "rng_stream": res["rng_stream"], "bytes_per_step": 2 * res["bytes_per_direction"]},
+                   "rng_stream": res["rng_stream"], "bytes_per_step": 2 * res["bytes_per_direction"],
+                   "bytes_counted": "algorithmic input + output bytes of both kernels",
+                   "buffer_sets": res["buffer_sets"],
+                   "timing": ("blocks of `steps` steps launched from the host" if args.eager or args.workload == "config5" else
+                              "blocks of `steps` steps recorded as one HIP graph and replayed") +
+                             " between two events, repeated for at least %.1f s" % args.min_seconds},
+        "timed_steps": res["timed_steps"],
         "frac_of_hbm_peak": res["gbs"] / HBM_PEAK_GBS,
-        "kernels": {"quantize": res["quantize"], "dequantize": res["dequantize"]},
+        "kernels": {k: {"us": res[k]["ms"] * 1e3, "gbs": res[k]["gbs"]} for k in ("quantize", "dequantize")},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get((args.workload, dom))},
     }
-    line["config"]["bytes_counted"] = "algorithmic input + output bytes of both kernels"
-    if args.workload == "config2":
-        r2, _ = run_workload(torch, "config2-2bit", args.steps, args.warmup)
-        line["two_bit_same_tensor"] = {"value": r2["gbs"], "unit": "GB/s", "ms_per_step": r2["ms_per_step"],
-                                       "frac_of_hbm_peak": r2["gbs"] / HBM_PEAK_GBS,
-                                       "kernels": {"quantize": r2["quantize"], "dequantize": r2["dequantize"]}}
-        torch.cuda.empty_cache()
-    if args.copy_calibration:
+    if args.copy_calibration and x is not None:
         y = torch.empty_like(x)
         for _ in range(20):
             y.copy_(x)
@@ -365,19 +402,23 @@ def main():
                                     "bytes_read": x.numel() * x.element_size(),
                                     "bytes_written": x.numel() * x.element_size()}
         del y
-    if args.all:
-        extra = []
-        for name in sorted(WORKLOADS):
-            if name == args.workload:
-                continue
-            r, _ = run_workload(torch, name, max(20, args.steps // 4), max(3, args.warmup // 4))
-            extra.append(r)
-            torch.cuda.empty_cache()
-        if args.workload != "config5":
-            extra.append(run_config5(torch, 20, 3))
+    if not args.only:
+        configs = {args.workload: compact(res)}
+        for name in BASELINE_SET + ["config5"]:
+            if name not in configs:
+                configs[name] = compact(run(name)[0])
+        # config 3 as BASELINE.json words it: the three BERT-large tensors of one layer, one after the other
+        parts = [configs[n] for n in ("config3-hidden", "config3-gelu", "config3-probs")]
+        c3_bytes = sum(p["bytes_per_direction"] for p in parts)
+        c3_us = sum(p["step"]["us"] for p in parts)
+        configs["config3"] = {"desc": "sum of config3-hidden (8 bit), config3-gelu (4 bit), config3-probs (2 bit)",
+                              "bytes_per_direction": c3_bytes,
+                              "step": {"us": c3_us, "gbs": 2 * c3_bytes / c3_us / 1e3,
+                                       "frac": 2 * c3_bytes / c3_us / 1e3 / HBM_PEAK_GBS}}
+        line["configs"] = configs
+        line["ceilings"] = run_ceilings(torch, timer)
         torch.cuda.empty_cache()
-        line["other_workloads"] = extra
-    if not args.no_cpu:
+    if not args.no_cpu and x is not None:
         line["cpu_baseline"] = cpu_baseline(torch, x, res["bits"], res["rng_stream"])
     else:
         line["cpu_baseline"] = None

@@ -109,16 +109,21 @@ __device__ __forceinline__ void rows_all_minmax(S& lo, S& hi) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Philox4x32-10.  The key schedule only depends on the seed, so it stays on the scalar unit; each
+// Philox4x32.  The key schedule only depends on the seed, so it stays on the scalar unit; each
 // round is two 32x32->64 multiplies and two three-input XORs (v_bitop3_b32, truth table 0x96).
+// Ten rounds for the reference's stream (cuRAND's generator); seven for the fast stream - the fewest
+// for which the generator's authors report that it passes BigCrush (Salmon et al., SC'11, table 2).
 // ------------------------------------------------------------------------------------------------
+#define PHILOX_REF_ROUNDS 10
+#define PHILOX_FAST_ROUNDS 7
 __device__ __forceinline__ uint32_t xor3(uint32_t a, uint32_t b, uint32_t c) {
   return __builtin_amdgcn_bitop3_b32(a, b, c, 0x96);
 }
-__device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
-                                              uint32_t k1, uint32_t (&out)[4]) {
+template <int ROUNDS>
+__device__ __forceinline__ void philox4x32(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                           uint32_t k1, uint32_t (&out)[4]) {
 #pragma unroll
-  for (int r = 0; r < 10; r++) {
+  for (int r = 0; r < ROUNDS; r++) {
     uint64_t p0 = (uint64_t)0xD2511F53u * c0;
     uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
     uint32_t n0 = xor3((uint32_t)(p1 >> 32), c1, k0);
@@ -167,14 +172,32 @@ __device__ __forceinline__ void stream_store(V v, V* p) {
 
 // round-to-nearest-even integer of z clamped below at 0: rint(max(z, 0)) of the reference's
 // __float2int_rn(fmax(z, 0)).  v_cvt_u32_f32 clamps negative inputs and NaN to 0, so no separate max is
-// needed; above 2^32 it saturates to 0xffffffff where the signed conversion saturates to 0x7fffffff -
-// the two agree in every bit the uint8 accumulator keeps once the code is shifted into its field.
+// needed.  From 2^31 on the reference's signed conversion saturates to 0x7fffffff: SAT = true reproduces
+// that (only min / max handed in by the caller can push a float code that far; with the group's own min
+// and max a code stays below 2^bits + 1), SAT = false leaves it out.
+template <bool SAT>
 __device__ __forceinline__ uint32_t rint_clamp0(float z) {
   float r = __builtin_rintf(z);
   uint32_t c;
   asm("v_cvt_u32_f32_e32 %0, %1" : "=v"(c) : "v"(r));
+  if (SAT) c = c < 0x7fffffffu ? c : 0x7fffffffu;
   return c;
 }
+
+// The same code taken from y directly, in two instructions instead of three, for 0 <= y < 2^22, negative y,
+// +-inf and NaN: y + (2^23 - 0.5) is rounded to a float whose unit in the last place is 1, i.e. to
+// 2^23 + rint(y - 0.5) (y - 0.5 itself is exact for 0.5 <= y < 2^23, so rounding the sum once equals
+// rounding the difference and then the integer; ties go to even in both since 2^23 is even), and the
+// integer sits in the low mantissa bits.  The median clamps to [2^23, 2^23 + 0x3fffff]: everything below
+// 0.5, negative or NaN gives 0 like the reference's fmax, and +inf (a half scale that overflowed) gives
+// low bits of all ones like the reference's saturated 0x7fffffff.  The bits above the code (0x4B...) never
+// reach the low 8 bits a byte keeps of a code shifted left by at most 7.
+__device__ __forceinline__ uint32_t clamp_code_bits(float w) {
+  float c;
+  asm("v_med3_f32 %0, %1, %2, %3" : "=v"(c) : "v"(w), "v"(8388608.0f), "v"(12582911.0f));
+  return __builtin_bit_cast(uint32_t, c);
+}
+__device__ __forceinline__ uint32_t code_bits_of(float y) { return clamp_code_bits(y + 8388607.5f); }
 
 // Correctly rounded c / s from the correctly rounded reciprocal r = RN(1/s) (Markstein): q = RN(c*r),
 // e = c - s*q exactly (one FMA), result RN(q + e*r).  Valid for finite nonzero s with a normal quotient;
@@ -242,17 +265,20 @@ template <> struct Elem<float> {
     float range = hi - lo;
     return (float)((double)(float)qmax / ((double)range + 2e-6));
   }
-  // code = rint(max(fma(x - mn, s, u) - 0.5, 0))
+  // code = rint(max(fma(x - mn, s, u) - 0.5, 0)).  ANY = true: min and scale may be anything (the pack entry
+  // point), the code is converted as the reference converts it; ANY = false: they are the group's own, the
+  // sum stays below 2^bits + 1 and the code is read off the float (code_bits_of: its low 8 bits count)
+  template <bool ANY>
   __device__ static __forceinline__ uint32_t code1(const Store& st, int k, int e, float mn, float s, float u) {
     float t = st.v[k][e] - mn;
     float y = __builtin_fmaf(t, s, u);
-    return rint_clamp0(y - 0.5f);
+    return ANY ? rint_clamp0<true>(y - 0.5f) : code_bits_of(y);
   }
-  template <bool CONST_NOISE>
+  template <bool CONST_NOISE, bool ANY>
   __device__ static __forceinline__ void codes(const Store& st, int k, float mn, float s, const float (&u)[4],
                                                uint32_t (&c)[4]) {
 #pragma unroll
-    for (int e = 0; e < 4; e++) c[e] = code1(st, k, e, mn, s, u[e]);
+    for (int e = 0; e < 4; e++) c[e] = code1<ANY>(st, k, e, mn, s, u[e]);
   }
 
   // ---- dequantize: out = float(code) / scale + min ----
@@ -364,14 +390,16 @@ template <> struct Elem<f16> {
     return y;
   }
   // half subtraction and half product (each rounded to half), then float: y = float(p) + u,
-  // code = rint(max(y - 0.5, 0))
+  // code = rint(max(y - 0.5, 0)).  |y| <= 65505 or y is infinite or NaN whatever min and scale are, so the
+  // code is always read off the float (code_bits_of); ANY changes nothing here.
+  template <bool ANY>
   __device__ static __forceinline__ uint32_t code1(const Store& st, int k, int e, f16 mn, f16 s, float u) {
     f16 t = st.v[k][e >> 1][e & 1] - mn;
     f16 p = t * s;
     float y = (float)p + u;
-    return rint_clamp0(y - 0.5f);
+    return code_bits_of(y);
   }
-  template <bool CONST_NOISE>
+  template <bool CONST_NOISE, bool ANY>
   __device__ static __forceinline__ void codes(const Store& st, int k, f16 mn, f16 s, const float (&u)[8],
                                                uint32_t (&c)[8]) {
     const f16x2 mn2 = {mn, mn}, s2 = {s, s};
@@ -380,13 +408,14 @@ template <> struct Elem<f16> {
       f16x2 t = st.v[k][j] - mn2;
       f16x2 p = t * s2;
       if (CONST_NOISE) {
-        // u = 0.5: float(p) + 0.5 and the following - 0.5 are both exact for every half p
-        // (at most 24 significant bits between 2^-1 and p's last bit), so y - 0.5 == float(p)
-        c[2 * j] = rint_clamp0((float)p.x);
-        c[2 * j + 1] = rint_clamp0((float)p.y);
+        // u = 0.5: float(p) + 0.5 and the following - 0.5 are both exact for every half p (at most 24
+        // significant bits between 2^-1 and p's last bit), so y - 0.5 == float(p) and the code is
+        // rint(float(p)): float(p) + 2^23 rounds to 2^23 + rint(float(p))
+        c[2 * j] = clamp_code_bits(widen_add_lo(p, 8388608.0f));
+        c[2 * j + 1] = clamp_code_bits(widen_add_hi(p, 8388608.0f));
       } else {
-        c[2 * j] = rint_clamp0(widen_add_lo(p, u[2 * j]) - 0.5f);
-        c[2 * j + 1] = rint_clamp0(widen_add_hi(p, u[2 * j + 1]) - 0.5f);
+        c[2 * j] = code_bits_of(widen_add_lo(p, u[2 * j]));
+        c[2 * j + 1] = code_bits_of(widen_add_hi(p, u[2 * j + 1]));
       }
     }
   }
@@ -465,16 +494,17 @@ template <> struct Elem<bf16> {
   __device__ static __forceinline__ float make_scale(float lo, float hi, int qmax) {
     return Elem<float>::make_scale(lo, hi, qmax);
   }
+  template <bool ANY>
   __device__ static __forceinline__ uint32_t code1(const Store& st, int k, int e, float mn, float s, float u) {
     float t = widen(st, k, e) - mn;
     float y = __builtin_fmaf(t, s, u);
-    return rint_clamp0(y - 0.5f);
+    return ANY ? rint_clamp0<true>(y - 0.5f) : code_bits_of(y);
   }
-  template <bool CONST_NOISE>
+  template <bool CONST_NOISE, bool ANY>
   __device__ static __forceinline__ void codes(const Store& st, int k, float mn, float s, const float (&u)[8],
                                                uint32_t (&c)[8]) {
 #pragma unroll
-    for (int e = 0; e < 8; e++) c[e] = code1(st, k, e, mn, s, u[e]);
+    for (int e = 0; e < 8; e++) c[e] = code1<ANY>(st, k, e, mn, s, u[e]);
   }
   __device__ static __forceinline__ bf16 finish(float q, float mn) { return (bf16)(q + mn); }
   __device__ static __forceinline__ uint32_t table_entry(float c, float s, float mn) {
@@ -551,7 +581,7 @@ __device__ __forceinline__ void fast_noise(int64_t n, int i, uint32_t k0, uint32
     for (int k = 0; k < CH; k++) {
       const uint64_t blk = (uint64_t)n * (GROUP / 8) + 16 * k + i;
       uint32_t r[4];
-      philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
+      philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
 #pragma unroll
       for (int e = 0; e < W; e++) u[k][e] = fast_piece(r[(e >> 2) * 2], r[(e >> 2) * 2 + 1], e & 3);
     }
@@ -562,7 +592,7 @@ __device__ __forceinline__ void fast_noise(int64_t n, int i, uint32_t k0, uint32
       // element block of (chunk, lane): (4*(16*chunk + lane)) / 8 = 8*chunk + lane/2
       const uint64_t blk = (uint64_t)n * (GROUP / 8) + 8 * (m + (odd ? 1 : 0)) + (i >> 1);
       uint32_t r[4];
-      philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
+      philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
       // the even lane owns elements 0..3 of a block (words 0,1), the odd lane elements 4..7 (words 2,3)
       const uint32_t ga = swap_with_neighbour(odd ? r[0] : r[2]);
       const uint32_t gb = swap_with_neighbour(odd ? r[1] : r[3]);
@@ -661,10 +691,10 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
         uint32_t r[4];
 #pragma unroll
         for (int ni = 0; ni < WPT; ni++) {
-          if ((ni & 3) == 0) philox4x32_10(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r);
+          if ((ni & 3) == 0) philox4x32<PHILOX_REF_ROUNDS>(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r);
           if (n0 + ni < N) {
             float u = curand_uniform_map(r[ni & 3]);
-            bytes[k][e] |= Elem<T>::code1(v[ni], k, e, lo_t[ni], s_t[ni], u) << (ni * BITS);
+            bytes[k][e] |= Elem<T>::template code1<GIVEN>(v[ni], k, e, lo_t[ni], s_t[ni], u) << (ni * BITS);
           }
         }
       }
@@ -690,7 +720,7 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
 #pragma unroll
         for (int k = 0; k < CH; k++) {
           uint32_t c[W];
-          Elem<T>::template codes<NOISE == GACT_NOISE_CONST>(v[ni], k, lo_t[ni], s_t[ni], u[k], c);
+          Elem<T>::template codes<NOISE == GACT_NOISE_CONST, GIVEN>(v[ni], k, lo_t[ni], s_t[ni], u[k], c);
 #pragma unroll
           for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (ni * BITS);
         }
@@ -1050,9 +1080,9 @@ __device__ __forceinline__ void quantize_supergroup_wide(const T* __restrict__ x
       uint32_t r[4];
 #pragma unroll
       for (int ni = 0; ni < WPT; ni++) {
-        if ((ni & 3) == 0) philox4x32_10(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r);
+        if ((ni & 3) == 0) philox4x32<PHILOX_REF_ROUNDS>(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r);
         if (n0 + ni < N)
-          bytes[e] |= Elem<T>::code1(v[ni], 0, e, lo_t[ni], s_t[ni], curand_uniform_map(r[ni & 3])) << (ni * BITS);
+          bytes[e] |= Elem<T>::template code1<false>(v[ni], 0, e, lo_t[ni], s_t[ni], curand_uniform_map(r[ni & 3])) << (ni * BITS);
       }
     }
   } else {
@@ -1064,7 +1094,7 @@ __device__ __forceinline__ void quantize_supergroup_wide(const T* __restrict__ x
         if (W == 8) {
           const uint64_t blk = (uint64_t)(n0 + g) * (GROUP / 8) + l;
           uint32_t r[4];
-          philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
+          philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
 #pragma unroll
           for (int e = 0; e < W; e++) u[0][e] = fast_piece(r[(e >> 2) * 2], r[(e >> 2) * 2 + 1], e & 3);
         } else {
@@ -1073,7 +1103,7 @@ __device__ __forceinline__ void quantize_supergroup_wide(const T* __restrict__ x
           const bool odd = l & 1;
           const uint64_t blk = (uint64_t)(n0 + g + (odd ? 1 : 0)) * (GROUP / 8) + (l >> 1);
           uint32_t r[4];
-          philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
+          philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
           const uint32_t ga = swap_with_neighbour(odd ? r[0] : r[2]);
           const uint32_t gb = swap_with_neighbour(odd ? r[1] : r[3]);
           const uint32_t a0 = odd ? ga : r[0], a1 = odd ? gb : r[1];   // group g
@@ -1100,7 +1130,7 @@ __device__ __forceinline__ void quantize_supergroup_wide(const T* __restrict__ x
         const int ni = g + h;
         if (n0 + ni < N) {
           uint32_t c[W];
-          Elem<T>::template codes<NOISE == GACT_NOISE_CONST>(v[ni], 0, lo_t[ni], s_t[ni], u[h], c);
+          Elem<T>::template codes<NOISE == GACT_NOISE_CONST, false>(v[ni], 0, lo_t[ni], s_t[ni], u[h], c);
 #pragma unroll
           for (int e = 0; e < W; e++) bytes[e] |= c[e] << (ni * BITS);
         }
@@ -1251,17 +1281,17 @@ pack_any_kernel(const T* __restrict__ data, const T* __restrict__ mn, const T* _
     if (NOISE == GACT_NOISE_INJECT) {
       u = noise[id];
     } else if (NOISE == GACT_NOISE_REF) {
-      if ((ni & 3) == 0) philox4x32_10(ni >> 2, 0u, (uint32_t)j, (uint32_t)((uint64_t)j >> 32), k0, k1, r);
+      if ((ni & 3) == 0) philox4x32<PHILOX_REF_ROUNDS>(ni >> 2, 0u, (uint32_t)j, (uint32_t)((uint64_t)j >> 32), k0, k1, r);
       u = curand_uniform_map(r[ni & 3]);
     } else if (NOISE == GACT_NOISE_FAST) {
       const uint64_t blk = (uint64_t)id >> 3;
-      philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
+      philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
       const int e = (int)(id & 7);
       u = fast_uniform_map((e & 1) ? (r[e >> 1] >> 16) : (r[e >> 1] & 0xffffu));
     }
     typename Elem<T>::Store one;
     Elem<T>::set(one, 0, 0, data[id]);
-    byte |= Elem<T>::code1(one, 0, 0, mn[sid], scale[sid], u) << (ni * bits);
+    byte |= Elem<T>::template code1<true>(one, 0, 0, mn[sid], scale[sid], u) << (ni * bits);
   }
   packed[j] = (uint8_t)byte;
 }
@@ -1319,12 +1349,12 @@ pack_rows8_kernel(const T* __restrict__ data, const T* __restrict__ mn, const T*
 #pragma unroll
       for (int e = 0; e < 8; e++) {
         const uint64_t j = (uint64_t)(j0 + e);
-        if ((ni & 3) == 0) philox4x32_10(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r[e]);
+        if ((ni & 3) == 0) philox4x32<PHILOX_REF_ROUNDS>(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r[e]);
         u[e] = curand_uniform_map(r[e][ni & 3]);
       }
     } else if (NOISE == GACT_NOISE_FAST) {
       const uint64_t blk = (uint64_t)id0 >> 3;
-      philox4x32_10(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r[0]);
+      philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r[0]);
 #pragma unroll
       for (int e = 0; e < 8; e++) u[e] = fast_uniform_map((e & 1) ? (r[0][e >> 1] >> 16) : (r[0][e >> 1] & 0xffffu));
     } else {
@@ -1335,7 +1365,7 @@ pack_rows8_kernel(const T* __restrict__ data, const T* __restrict__ mn, const T*
     for (int e = 0; e < 8; e++) {
       typename Elem<T>::Store one;
       Elem<T>::set(one, 0, 0, x[e]);
-      bytes[e] |= Elem<T>::code1(one, 0, 0, lo, sc, u[e]) << (ni * bits);
+      bytes[e] |= Elem<T>::template code1<true>(one, 0, 0, lo, sc, u[e]) << (ni * bits);
     }
   }
   u32x2 w;
@@ -1675,27 +1705,72 @@ calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, cons
 // ------------------------------------------------------------------------------------------------
 // Batched launch over a table of tensors with device-resident bits.
 // ------------------------------------------------------------------------------------------------
-// One wave: lane l sizes tensors l, l+64, ...; a running offset is carried across rounds of 64 with a
-// wave-wide inclusive scan.  plan[0] = arena bytes needed, plan[1] = ok flag, plan[2 + k] = number of
-// tensors at width 1 << k (the work kernels of a width nobody uses leave at once).
+// The workspace of a batched launch (device memory the caller brings, or the library's static array):
+//   BatchHeader                      what the plan found
+//   int32 tensor_class_off[L]        blocks of earlier tensors of the same class
+//   int32 block_tensor[total_blocks] tensor of every block of the grid (dequantize: one launch over all blocks)
+//   int32x2 class_list[total_blocks] the blocks sorted by class, as (tensor, block within the tensor): the quantize
+//                                    kernel of a class walks its own stretch of this list and nothing else
+// A class is an (element type, width) pair: 3 types x 4 widths.
+#define BATCH_CLASSES 12
+struct BatchHeader {
+  int64_t need;                        // arena bytes the table needs
+  int64_t ok;                          // 1: every width valid and need <= capacity
+  int64_t tensors_at[4];               // tensors at width 1, 2, 4, 8
+  int64_t reserved[2];
+  int64_t class_count[BATCH_CLASSES];  // blocks per class
+  int64_t class_start[BATCH_CLASSES];  // first entry of the class in class_list
+};
+static_assert(sizeof(BatchHeader) == 256, "the header is 32 int64");
+struct BatchWorkspace {
+  BatchHeader* hdr;
+  int32_t* tensor_class_off;
+  int32_t* block_tensor;
+  int2* class_list;
+};
+__host__ __device__ inline int64_t batch_workspace_need(int64_t L, int64_t total_blocks) {
+  return (int64_t)sizeof(BatchHeader) + ((L + 63) / 64 * 64) * 4 + ((total_blocks + 1) / 2 * 2) * 4 + total_blocks * 8;
+}
+__host__ __device__ inline BatchWorkspace batch_workspace(void* base, int64_t L, int64_t total_blocks) {
+  BatchWorkspace w;
+  uint8_t* p = (uint8_t*)base;
+  w.hdr = (BatchHeader*)p;
+  w.tensor_class_off = (int32_t*)(p + sizeof(BatchHeader));
+  w.block_tensor = w.tensor_class_off + (L + 63) / 64 * 64;
+  w.class_list = (int2*)(w.block_tensor + (total_blocks + 1) / 2 * 2);  // stays 8-byte aligned
+  return w;
+}
+__device__ __forceinline__ int width_index(int bits) { return bits == 1 ? 0 : bits == 2 ? 1 : bits == 4 ? 2 : 3; }
+
+// One wave: lane l sizes tensors l, l+64, ...; running offsets are carried across rounds of 64 with wave-wide
+// inclusive scans - one for the packed-arena offsets, one per class for the position of a tensor's blocks
+// among the blocks of its class.
 __global__ void __launch_bounds__(64)
 batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int L, int64_t capacity,
-                  int64_t* plan) {
+                  BatchWorkspace ws) {
   const int lane = threadIdx.x;
   int64_t base = 0;
   int bad = 0;
   int cnt[4] = {0, 0, 0, 0};
+  int class_base[BATCH_CLASSES];
+#pragma unroll
+  for (int c = 0; c < BATCH_CLASSES; c++) class_base[c] = 0;
   for (int t0 = 0; t0 < L; t0 += 64) {
     const int t = t0 + lane;
     int64_t bytes = 0;
+    int cls = -1, nb = 0;
     if (t < L) {
       int bt = bits[t];
       if (!(bt == 1 || bt == 2 || bt == 4 || bt == 8)) { bad = 1; bt = 8; }
-      cnt[bt == 1 ? 0 : bt == 2 ? 1 : bt == 4 ? 2 : 3]++;
+      int dt = table[t].dtype;
+      if (dt < 0 || dt > 2) { bad = 1; dt = 0; }
+      cnt[width_index(bt)]++;
+      cls = dt * 4 + width_index(bt);
       const int wpt = 8 / bt;
       const int64_t N = (table[t].numel + GROUP - 1) / GROUP;
       const int64_t n_round = (N + wpt - 1) / wpt * wpt;
       bytes = ((int64_t)bt * n_round * (GROUP / 8) + 255) / 256 * 256;
+      nb = (int)((N + 127) / 128);
     }
     int64_t incl = bytes;
 #pragma unroll
@@ -1705,6 +1780,18 @@ batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int
     }
     if (t < L) table[t].packed_offset = base + incl - bytes;
     base += __shfl(incl, 63, 64);
+#pragma unroll
+    for (int c = 0; c < BATCH_CLASSES; c++) {
+      const int v = cls == c ? nb : 0;
+      int in = v;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(in, off, 64);
+        if (lane >= off) in += up;
+      }
+      if (cls == c) ws.tensor_class_off[t] = class_base[c] + in - v;
+      class_base[c] += __shfl(in, 63, 64);
+    }
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) {
@@ -1713,10 +1800,18 @@ batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int
     for (int k = 0; k < 4; k++) cnt[k] += __shfl_xor(cnt[k], off, 64);
   }
   if (lane == 0) {
-    plan[0] = base;
-    plan[1] = (!bad && base <= capacity) ? 1 : 0;
+    ws.hdr->need = base;
+    ws.hdr->ok = (!bad && base <= capacity) ? 1 : 0;
 #pragma unroll
-    for (int k = 0; k < 4; k++) plan[2 + k] = cnt[k];
+    for (int k = 0; k < 4; k++) ws.hdr->tensors_at[k] = cnt[k];
+    ws.hdr->reserved[0] = ws.hdr->reserved[1] = 0;
+    int64_t run = 0;
+#pragma unroll
+    for (int c = 0; c < BATCH_CLASSES; c++) {
+      ws.hdr->class_count[c] = class_base[c];
+      ws.hdr->class_start[c] = run;
+      run += class_base[c];
+    }
   }
 }
 
@@ -1729,27 +1824,45 @@ __device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ t
   return lo;
 }
 
-// Quantize, one launch per width and element type: blocks whose tensor has another width or type leave at once,
-// so every combination gets a kernel with its own register allocation (176 registers at 1 bit float, 117 at
-// 1 bit half, 34 at 8 bit half).
+// One thread per block of the grid: find its tensor, note it, and enter the block in its class's stretch of
+// the list.  Runs after the plan kernel on the same stream.
+__global__ void __launch_bounds__(256)
+batch_lists_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
+                   int64_t total_blocks, BatchWorkspace ws) {
+  const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (g >= total_blocks) return;
+  const int t = batch_find(table, L, g);
+  int bt = bits[t];
+  if (!(bt == 1 || bt == 2 || bt == 4 || bt == 8)) bt = 8;   // as the plan counted it; the launch is void anyway
+  int dt = table[t].dtype;
+  if (dt < 0 || dt > 2) dt = 0;
+  const int cls = dt * 4 + width_index(bt);
+  const int local = (int)(g - table[t].first_block);
+  ws.block_tensor[g] = t;
+  ws.class_list[ws.hdr->class_start[cls] + ws.tensor_class_off[t] + local] = make_int2(t, local);
+}
+
+// Quantize, one launch per width and element type, so that every combination gets a kernel with its own
+// register allocation (176 registers at 1 bit float, 117 at 1 bit half, 34 at 8 bit half).  The workgroups
+// of a launch stride over the blocks of their class: the grid need not know how many there are.
 template <typename T, int BITS, int NOISE>
 __global__ void __launch_bounds__(256)
-quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
-                        const int64_t* __restrict__ plan, const int32_t* __restrict__ block_map,
+quantize_batched_kernel(const gact_batch_entry* __restrict__ table, BatchWorkspace ws,
                         uint8_t* __restrict__ packed_arena, uint8_t* __restrict__ scale_arena,
                         uint8_t* __restrict__ min_arena) {
-  // the plan did not fit the arena or held an invalid width, or no tensor has this width
-  if (plan[1] == 0 || plan[2 + (BITS == 1 ? 0 : BITS == 2 ? 1 : BITS == 4 ? 2 : 3)] == 0) return;
-  const int64_t block = blockIdx.x;  // the XCD-aware order gains nothing here (800 -> 797 us on 120 half tensors)
-  const int t = block_map ? block_map[block] : batch_find(table, L, block);
-  if (bits[t] != BITS) return;
-  const gact_batch_entry ent = table[t];
-  if (ent.dtype != Elem<T>::kDtype) return;
-  const int64_t N = (ent.numel + GROUP - 1) / GROUP;
-  const int64_t lb = block - ent.first_block;
-  quantize_block128<T, BITS, NOISE>((const T*)ent.x, ent.numel, N, lb, packed_arena + ent.packed_offset,
-                                    (typename Elem<T>::Stat*)(scale_arena + ent.stats_offset * 4),
-                                    (T*)(min_arena + ent.stats_offset * 4), ent.seed);
+  if (ws.hdr->ok == 0) return;  // the plan did not fit the arena or held an invalid width
+  constexpr int CLS = Elem<T>::kDtype * 4 + (BITS == 1 ? 0 : BITS == 2 ? 1 : BITS == 4 ? 2 : 3);
+  const int64_t count = ws.hdr->class_count[CLS];
+  const int2* __restrict__ list = ws.class_list + ws.hdr->class_start[CLS];
+#pragma unroll 1
+  for (int64_t b = blockIdx.x; b < count; b += gridDim.x) {
+    const int2 e = list[b];
+    const gact_batch_entry ent = table[e.x];
+    const int64_t N = (ent.numel + GROUP - 1) / GROUP;
+    quantize_block128<T, BITS, NOISE>((const T*)ent.x, ent.numel, N, e.y, packed_arena + ent.packed_offset,
+                                      (typename Elem<T>::Stat*)(scale_arena + ent.stats_offset * 4),
+                                      (T*)(min_arena + ent.stats_offset * 4), ent.seed);
+  }
 }
 
 // Dequantize, one launch for all widths (every width fits 60 registers): the width of a block's tensor is read
@@ -1767,16 +1880,15 @@ __device__ __forceinline__ void dequantize_batched_block(const gact_batch_entry&
 }
 // grid: two workgroups per block of 128 groups
 __global__ void __launch_bounds__(256)
-dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
-                          const int64_t* __restrict__ plan, const int32_t* __restrict__ block_map,
-                          const uint8_t* __restrict__ packed_arena, const uint8_t* __restrict__ scale_arena,
-                          const uint8_t* __restrict__ min_arena) {
-  if (plan[1] == 0) return;
+dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits,
+                          BatchWorkspace ws, const uint8_t* __restrict__ packed_arena,
+                          const uint8_t* __restrict__ scale_arena, const uint8_t* __restrict__ min_arena) {
+  if (ws.hdr->ok == 0) return;
   // half a block is the single-tensor kernel's tile; same XCD-aware order (715 -> 709 us on 120 half tensors)
   const uint32_t tile = xcd_tile<GACT_XCD_RUN_DQ>(blockIdx.x, gridDim.x);
   const int64_t block = tile >> 1;
   const int half = tile & 1;
-  const int t = block_map ? block_map[block] : batch_find(table, L, block);
+  const int t = ws.block_tensor[block];
   const gact_batch_entry ent = table[t];
   const int64_t lb = block - ent.first_block;
   const uint8_t* packed = packed_arena + ent.packed_offset;
@@ -2207,31 +2319,33 @@ int gact_calc_precision_device(int32_t* b, const float* C, const int64_t* w, int
   return launch_status();
 }
 
-int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t capacity, int64_t* plan,
-                    void* stream) {
-  if (L < 0 || L > (1 << 30) || capacity < 0) return GACT_EINVAL;
-  if (!plan) return GACT_EINVAL;
-  if (L > 0 && (!table || !bits)) return GACT_EINVAL;
-  hipLaunchKernelGGL(batch_plan_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, table, bits, (int)L, capacity, plan);
+int64_t gact_batch_workspace_bytes(int64_t L, int64_t total_blocks) {
+  if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x3fffffffLL) return GACT_EINVAL;
+  return batch_workspace_need(L, total_blocks);
+}
+
+namespace {
+int batch_plan_on(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks, int64_t capacity,
+                  void* workspace, hipStream_t s) {
+  const BatchWorkspace ws = batch_workspace(workspace, L, total_blocks);
+  hipLaunchKernelGGL(batch_plan_kernel, dim3(1), dim3(64), 0, s, table, bits, (int)L, capacity, ws);
+  if (total_blocks > 0)
+    hipLaunchKernelGGL(batch_lists_kernel, dim3((unsigned)((total_blocks + 255) / 256)), dim3(256), 0, s, table, bits, (int)L,
+                       total_blocks, ws);
   return launch_status();
 }
 
-int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
-                          int noise_mode, int dtypes, const int64_t* plan, const int32_t* block_map,
-                          void* packed_arena, void* scale_arena, void* min_arena, void* stream) {
-  if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x7fffffffLL) return GACT_EINVAL;
-  if (noise_mode != GACT_NOISE_CONST && noise_mode != GACT_NOISE_REF && noise_mode != GACT_NOISE_FAST)
-    return GACT_EINVAL;  // injected noise is a single-tensor test mode
-  if (dtypes < 0 || dtypes > GACT_DTYPES_ALL) return GACT_EINVAL;
-  if (dtypes == 0) dtypes = GACT_DTYPES_ALL;
-  if (L == 0 || total_blocks == 0) return GACT_OK;
-  if (!table || !bits || !plan || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
-  if (!aligned16(packed_arena)) return GACT_EALIGN;
-  const dim3 grid((unsigned)total_blocks), block(256);
-  hipStream_t s = (hipStream_t)stream;
+int quantize_batched_on(const gact_batch_entry* table, int64_t L, int64_t total_blocks, int noise_mode, int dtypes,
+                        void* workspace, void* packed_arena, void* scale_arena, void* min_arena, hipStream_t s) {
+  const BatchWorkspace ws = batch_workspace(workspace, L, total_blocks);
+  // the widths live on the device, so a launch cannot be sized to its class: a quarter of the blocks (all of
+  // them when there are few), striding over the class's list, keeps the chip full and the empty classes cheap
+  int64_t g = total_blocks / 4;
+  if (g < 8192) g = total_blocks < 8192 ? total_blocks : 8192;
+  const dim3 grid((unsigned)g), block(256);
 #define GACT_LAUNCH_QB(T, B, M)                                                                               \
-  hipLaunchKernelGGL((quantize_batched_kernel<T, B, M>), grid, block, 0, s, table, bits, (int)L, plan,       \
-                     block_map, (uint8_t*)packed_arena, (uint8_t*)scale_arena, (uint8_t*)min_arena)
+  hipLaunchKernelGGL((quantize_batched_kernel<T, B, M>), grid, block, 0, s, table, ws, (uint8_t*)packed_arena, \
+                     (uint8_t*)scale_arena, (uint8_t*)min_arena)
 #define GACT_LAUNCH_QB_ALL(M)                                                                                 \
   do {                                                                                                        \
     if (dtypes & GACT_DTYPES_F32) {                                                                           \
@@ -2257,16 +2371,46 @@ int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, in
   return launch_status();
 }
 
-int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
-                            const int64_t* plan, const int32_t* block_map, const void* packed_arena,
-                            const void* scale_arena, const void* min_arena, void* stream) {
-  if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x3fffffffLL) return GACT_EINVAL;
+inline int batched_args_ok(int64_t L, int64_t total_blocks) {
+  return !(L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x3fffffffLL);
+}
+}  // namespace
+
+int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks, int64_t capacity,
+                    void* workspace, void* stream) {
+  if (!batched_args_ok(L, total_blocks) || capacity < 0) return GACT_EINVAL;
+  if (!workspace) return GACT_EINVAL;
+  if (!aligned16(workspace)) return GACT_EALIGN;
+  if (L > 0 && (!table || !bits)) return GACT_EINVAL;
+  return batch_plan_on(table, bits, L, total_blocks, capacity, workspace, (hipStream_t)stream);
+}
+
+int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
+                          int noise_mode, int dtypes, const void* workspace, void* packed_arena, void* scale_arena,
+                          void* min_arena, void* stream) {
+  if (!batched_args_ok(L, total_blocks)) return GACT_EINVAL;
+  if (noise_mode != GACT_NOISE_CONST && noise_mode != GACT_NOISE_REF && noise_mode != GACT_NOISE_FAST)
+    return GACT_EINVAL;  // injected noise is a single-tensor test mode
+  if (dtypes < 0 || dtypes > GACT_DTYPES_ALL) return GACT_EINVAL;
+  if (dtypes == 0) dtypes = GACT_DTYPES_ALL;
   if (L == 0 || total_blocks == 0) return GACT_OK;
-  if (!table || !bits || !plan || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
-  if (!aligned16(packed_arena)) return GACT_EALIGN;
+  if (!table || !bits || !workspace || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
+  if (!aligned16(packed_arena) || !aligned16(workspace)) return GACT_EALIGN;
+  return quantize_batched_on(table, L, total_blocks, noise_mode, dtypes, const_cast<void*>(workspace), packed_arena,
+                             scale_arena, min_arena, (hipStream_t)stream);
+}
+
+int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
+                            const void* workspace, const void* packed_arena, const void* scale_arena,
+                            const void* min_arena, void* stream) {
+  if (!batched_args_ok(L, total_blocks)) return GACT_EINVAL;
+  if (L == 0 || total_blocks == 0) return GACT_OK;
+  if (!table || !bits || !workspace || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
+  if (!aligned16(packed_arena) || !aligned16(workspace)) return GACT_EALIGN;
   const dim3 grid((unsigned)(2 * total_blocks)), block(256);
-  hipLaunchKernelGGL(dequantize_batched_kernel, grid, block, 0, (hipStream_t)stream, table, bits, (int)L, plan, block_map,
-                     (const uint8_t*)packed_arena, (const uint8_t*)scale_arena, (const uint8_t*)min_arena);
+  hipLaunchKernelGGL(dequantize_batched_kernel, grid, block, 0, (hipStream_t)stream, table, bits,
+                     batch_workspace(const_cast<void*>(workspace), L, total_blocks), (const uint8_t*)packed_arena,
+                     (const uint8_t*)scale_arena, (const uint8_t*)min_arena);
   return launch_status();
 }
 

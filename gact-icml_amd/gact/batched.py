@@ -2,9 +2,10 @@
 
 The reference quantizes one tensor per call (gact/gact/quantizer.py:95-142) and computes the widths on
 the host (gact/gact/autoprec.py:188-209).  Here ``calc_precision_device`` leaves the widths in device
-memory, a one-thread planning kernel turns them into packed-arena offsets, and a single grid then
-quantizes (or dequantizes) every tensor at its own width.  Nothing is read back to the host; the
-results are identical to calling ``op_quantize`` / ``op_dequantize`` tensor by tensor.
+memory, a planning step (two small kernels) turns them into packed-arena offsets and into a list of the
+grid's blocks sorted by width, and the batched kernels then quantize (one launch per width, each over its
+own blocks) or dequantize (one launch) every tensor at its own width.  Nothing is read back to the host;
+the results are identical to calling ``op_quantize`` / ``op_dequantize`` tensor by tensor.
 
 Grid layout: a block owns 128 groups of 256 elements whatever the width, so the grid
 (sum over tensors of ceil(N_i/128) blocks) is known on the host without knowing the widths.
@@ -17,23 +18,35 @@ GROUPS_PER_BLOCK = 128
 
 
 class BatchedPacked:
-    """What a batched quantize leaves behind: the arenas, the table and the per-tensor geometry."""
+    """What a batched quantize leaves behind: the arenas, the table and the per-tensor geometry.
 
-    def __init__(self, owner, packed, scale, mn, table, bits, plan, shapes, dtypes, seeds):
+    The widths come from device memory, so whether they were all valid (1, 2, 4 or 8 - a tensor that
+    calc_precision left at 32 is not) and whether the arena was large enough is only known on the
+    device: when either fails the kernels write nothing.  ``ok()`` reads that verdict back (it
+    synchronises); ``per_tensor`` and ``BatchedQuantizer.dequantize`` call it and raise."""
+
+    def __init__(self, owner, packed, scale, mn, table, bits, workspace, shapes, dtypes, seeds):
         self.owner = owner
         self.seeds = list(seeds)
         self.packed, self.scale, self.min = packed, scale, mn
-        self.table, self.bits, self.plan = table, bits, plan
+        self.table, self.bits, self.workspace = table, bits, workspace
         self.shapes, self.dtypes = shapes, dtypes
 
     def ok(self):
-        """Synchronising check that the plan fitted the arena and every width was valid."""
-        vals = self.plan.tolist()
+        """(plan succeeded, arena bytes the table needs); synchronises."""
+        vals = self.workspace[:16].view(torch.int64).tolist()
         return bool(vals[1]), vals[0]
+
+    def require_ok(self):
+        good, need = self.ok()
+        if not good:
+            raise RuntimeError("gact: the batched launch was void - a width outside {1, 2, 4, 8} or a packed arena "
+                               "of %d bytes where %d are needed; nothing was quantized" % (self.packed.numel(), need))
 
     def per_tensor(self, i):
         """Views (packed bytes, bits, scale[N,1,1], min[N,1,1]) of tensor i in op_quantize's format.
         Reads the width and the offset back from the device (synchronises)."""
+        self.require_ok()
         b = int(self.bits[i].item())
         numel = self.owner.numels[i]
         N = (numel + _abi.GROUP - 1) // _abi.GROUP
@@ -57,7 +70,7 @@ class BatchedQuantizer:
         self.device = torch.device(device)
         self.numels = [int(n) for n in numels]
         self.dtypes = list(dtypes)
-        # which element types occur (bit 0 float, bit 1 half): the library launches only their kernels
+        # which element types occur (bit 0 float, bit 1 half, bit 2 bfloat16): the library launches only their kernels
         self.dtype_mask = 0
         for dt in self.dtypes:
             self.dtype_mask |= 1 << _abi.dtype_code(dt)
@@ -73,12 +86,7 @@ class BatchedQuantizer:
             groups += (N + 7) // 8 * 8   # 32-byte aligned rows: the dequantize kernel reads them 16 bytes at a time
         self.total_blocks = blocks
         self.total_groups = groups
-        # block -> tensor, fixed by the geometry: lets a block find its tensor with one load
-        bm = torch.empty((max(blocks, 1),), dtype=torch.int32)
-        for i in range(self.L):
-            end = self.first_blocks[i + 1] if i + 1 < self.L else blocks
-            bm[self.first_blocks[i]:end] = i
-        self.block_map = bm.to(self.device)
+        self.workspace_bytes = int(_abi.lib().gact_batch_workspace_bytes(self.L, self.total_blocks))
 
     # ---- arena sizing (host-side bounds; the exact need is computed on the device) ----
     def arena_bytes_for_budget(self, target_bits):
@@ -91,6 +99,14 @@ class BatchedQuantizer:
     def arena_bytes_worst_case(self):
         """Every tensor at 8 bits."""
         return sum(self.numels) + 768 * self.L + 256
+
+    def new_workspace(self):
+        """Device memory a plan of this geometry fills (header, block -> tensor map, blocks sorted by kind)."""
+        return torch.empty((self.workspace_bytes,), dtype=torch.uint8, device=self.device)
+
+    def plan_ok(self, workspace):
+        """Whether the last plan written to this workspace succeeded; synchronises."""
+        return bool(workspace[8:16].view(torch.int64).item())
 
     def _table(self, tensors, seeds):
         arr = (_abi.BatchEntry * self.L)()
@@ -112,49 +128,63 @@ class BatchedQuantizer:
         host = torch.frombuffer(bytearray(bytes(arr)), dtype=torch.uint8)
         return host.to(self.device, non_blocking=False)
 
+    # ---- the launches on caller-owned buffers (nothing is allocated, nothing synchronises) ----
+    def launch_quantize(self, table, bits, packed, scale, mn, workspace, mode):
+        """Plan into `workspace` from the device-resident `bits`, then quantize every tensor of `table`."""
+        lib = _abi.lib()
+        st = torch.cuda.current_stream(self.device).cuda_stream
+        _abi.check(lib.gact_batch_plan(table.data_ptr(), bits.data_ptr(), self.L, self.total_blocks, packed.numel(),
+                                       workspace.data_ptr(), st))
+        _abi.check(lib.gact_quantize_batched(table.data_ptr(), bits.data_ptr(), self.L, self.total_blocks, mode,
+                                             self.dtype_mask, workspace.data_ptr(), packed.data_ptr(),
+                                             scale.data_ptr(), mn.data_ptr(), st))
+
+    def launch_dequantize(self, table, bits, packed, scale, mn, workspace):
+        """Plan into `workspace` (the table's x point at the outputs; planning again from the same widths gives
+        the same offsets without reading anything back), then dequantize every tensor."""
+        lib = _abi.lib()
+        st = torch.cuda.current_stream(self.device).cuda_stream
+        _abi.check(lib.gact_batch_plan(table.data_ptr(), bits.data_ptr(), self.L, self.total_blocks, packed.numel(),
+                                       workspace.data_ptr(), st))
+        _abi.check(lib.gact_dequantize_batched(table.data_ptr(), bits.data_ptr(), self.L, self.total_blocks,
+                                               workspace.data_ptr(), packed.data_ptr(), scale.data_ptr(),
+                                               mn.data_ptr(), st))
+
     def quantize(self, tensors, bits, seeds, arena_bytes=None, rng_stream=None):
-        """Quantize all tensors in one launch.  `bits` is an int32 tensor on the device (e.g. the output
-        of calc_precision_device).  Returns a BatchedPacked; nothing synchronises."""
+        """Quantize all tensors in one batched launch.  `bits` is an int32 tensor on the device (e.g. the output
+        of calc_precision_device) holding 1, 2, 4 or 8 for every tensor.  Returns a BatchedPacked; nothing
+        synchronises, so a void launch (see BatchedPacked) shows when the result is used."""
         from .cpp_extension.quantization import _noise_mode
         if bits.dtype != torch.int32 or not bits.is_cuda or bits.numel() != self.L:
             raise RuntimeError("bits must be an int32 CUDA tensor with one entry per tensor")
         mode = _noise_mode(None, rng_stream)
         if arena_bytes is None:
             arena_bytes = self.arena_bytes_worst_case()
-        lib = _abi.lib()
         with torch.cuda.device(self.device):
             table = self._table(tensors, seeds)
             packed = torch.empty((int(arena_bytes),), dtype=torch.uint8, device=self.device)
             scale = torch.empty((self.total_groups * 4,), dtype=torch.uint8, device=self.device)
             mn = torch.empty((self.total_groups * 4,), dtype=torch.uint8, device=self.device)
-            plan = torch.empty((6,), dtype=torch.int64, device=self.device)
-            st = torch.cuda.current_stream(self.device).cuda_stream
-            _abi.check(lib.gact_batch_plan(table.data_ptr(), bits.data_ptr(), self.L, packed.numel(),
-                                           plan.data_ptr(), st))
-            _abi.check(lib.gact_quantize_batched(table.data_ptr(), bits.data_ptr(), self.L, self.total_blocks, mode,
-                                                 self.dtype_mask, plan.data_ptr(), self.block_map.data_ptr(),
-                                                 packed.data_ptr(),
-                                                 scale.data_ptr(), mn.data_ptr(), st))
-        # the widths are kept as they were at quantize time: the caller may refresh its own copy
-        return BatchedPacked(self, packed, scale, mn, table, bits.clone(), plan, [t.shape for t in tensors],
+            ws = self.new_workspace()
+            # the widths are kept as they were at quantize time: the caller may refresh its own copy
+            kept = bits.clone()
+            self.launch_quantize(table, kept, packed, scale, mn, ws, mode)
+        return BatchedPacked(self, packed, scale, mn, table, kept, ws, [t.shape for t in tensors],
                              list(self.dtypes), seeds)
 
-    def dequantize(self, q, outs=None):
-        """Dequantize every tensor of a BatchedPacked in one launch into fresh tensors (or `outs`)."""
-        lib = _abi.lib()
+    def dequantize(self, q, outs=None, check=True):
+        """Dequantize every tensor of a BatchedPacked in one launch into fresh tensors (or `outs`).
+        check = True reads the plan's verdict back first (one synchronisation) and raises when the quantize
+        launch was void; pass False where nothing may synchronise (stream capture) and the caller has
+        checked ``q.ok()`` itself."""
+        if check:
+            q.require_ok()
         with torch.cuda.device(self.device):
             if outs is None:
                 outs = [torch.empty(s, dtype=d, device=self.device) for s, d in zip(q.shapes, q.dtypes)]
-            # a fresh table with x pointing at the outputs; planning it again from the same widths gives
-            # the same offsets without reading anything back
             table = self._table(outs, q.seeds)
-            plan = torch.empty((6,), dtype=torch.int64, device=self.device)
-            st = torch.cuda.current_stream(self.device).cuda_stream
-            _abi.check(lib.gact_batch_plan(table.data_ptr(), q.bits.data_ptr(), self.L, q.packed.numel(),
-                                           plan.data_ptr(), st))
-            _abi.check(lib.gact_dequantize_batched(table.data_ptr(), q.bits.data_ptr(), self.L, self.total_blocks,
-                                                   plan.data_ptr(), self.block_map.data_ptr(), q.packed.data_ptr(),
-                                                   q.scale.data_ptr(), q.min.data_ptr(), st))
+            ws = self.new_workspace()
+            self.launch_dequantize(table, q.bits, q.packed, q.scale, q.min, ws)
             # keep the table alive until the stream has consumed it
-            q._dq_table = (table, plan)
+            q._dq_table = (table, ws)
         return outs

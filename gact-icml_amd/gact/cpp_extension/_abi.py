@@ -15,7 +15,7 @@ F32, F16, BF16 = 0, 1, 2
 NOISE_CONST, NOISE_INJECT, NOISE_REF, NOISE_FAST = 0, 1, 2, 3
 NOISE_MODES = {"deterministic": NOISE_CONST, "inject": NOISE_INJECT, "reference": NOISE_REF, "fast": NOISE_FAST}
 GROUP = 256
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 class BatchEntry(ctypes.Structure):
@@ -50,9 +50,10 @@ SIGNATURES = {
     "gact_mask_unpack": (_i32, [_vp, _i64, _vp, _vp]),
     "gact_calc_precision": (_i32, [_vp, _vp, _vp, _i64, _f64]),
     "gact_calc_precision_device": (_i32, [_vp, _vp, _vp, _i64, _f64, _vp, _vp]),
-    "gact_batch_plan": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp]),
-    "gact_quantize_batched": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),
-    "gact_dequantize_batched": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "gact_batch_workspace_bytes": (_i64, [_i64, _i64]),
+    "gact_batch_plan": (_i32, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
+    "gact_quantize_batched": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
+    "gact_dequantize_batched": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
 }
 
 

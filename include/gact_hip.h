@@ -17,7 +17,7 @@
 extern "C" {
 #endif
 
-#define GACT_ABI_VERSION 4
+#define GACT_ABI_VERSION 5
 
 /* element types of activations, min, max and scale */
 #define GACT_F32 0
@@ -33,7 +33,7 @@ extern "C" {
 #define GACT_NOISE_INJECT 1 /* u read from a float tensor laid out like the (padded) data        */
 #define GACT_NOISE_REF 2    /* the reference's stream: one Philox4x32-10 state per output byte,  */
                             /* (seed, subsequence = byte index, offset 0), cuRAND uniform map    */
-#define GACT_NOISE_FAST 3   /* one Philox4x32-10 block per 8 consecutive elements, 16-bit noise  */
+#define GACT_NOISE_FAST 3   /* one Philox4x32-7 block per 8 consecutive elements, 16-bit noise   */
 
 #define GACT_OK 0
 #define GACT_EINVAL (-1) /* bad argument (bits not in {1,2,4,8}, negative size, null pointer ...) */
@@ -118,35 +118,39 @@ typedef struct gact_batch_entry {
   int64_t stats_offset;  /* element offset of this tensor's scale/min rows in the stats arenas      */
 } gact_batch_entry;
 
-/* Fill packed_offset (256-byte aligned, in table order) from device-resident bits.  `plan` is a device
- * array of six int64: plan[0] receives the arena bytes the table needs, plan[1] receives 1 when every
- * bits[i] is in {1,2,4,8} and plan[0] <= capacity, else 0 (the batched kernels then do nothing),
- * plan[2..5] the number of tensors at width 1, 2, 4, 8.  No counterpart in the reference. */
-int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t capacity, int64_t* plan,
-                    void* stream);
+/* Bytes of device workspace gact_batch_plan fills for a table of L tensors whose grid has total_blocks
+ * blocks (the sum of ceil(N_i/128): a block is 128 groups whatever the width).  16-byte aligned memory. */
+int64_t gact_batch_workspace_bytes(int64_t L, int64_t total_blocks);
 
-/* Quantize / dequantize all L tensors of the table over a grid of `total_blocks` blocks (the sum of
- * ceil(N_i/128)), each tensor at its own bits[i] read from device memory (quantize launches the grid once
- * per width, blocks of tensors at another width leave at once; dequantize is one launch).  Scale and min of tensor i
+/* Plan a batched launch from device-resident bits: fills packed_offset of every table entry (256-byte
+ * aligned, in table order) and the workspace - a header of 32 int64 ([0] the arena bytes the table needs,
+ * [1] 1 when every bits[i] is in {1,2,4,8}, every dtype is known and [0] <= capacity, else 0: the batched
+ * kernels then do nothing, [2..5] the number of tensors at width 1, 2, 4, 8), the tensor of every block, and
+ * the blocks sorted by (element type, width), which is what lets each quantize kernel visit only the blocks
+ * of its own kind.  Two small kernels; nothing is read back.  No counterpart in the reference. */
+int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
+                    int64_t capacity, void* workspace, void* stream);
+
+/* Quantize / dequantize all L tensors of the table, each at its own bits[i] read from device memory
+ * (quantize launches one kernel per width and element type, whose workgroups stride over the blocks of that
+ * kind in the workspace's list; dequantize is one launch over all blocks).  Scale and min of tensor i
  * are written at byte offset 4*stats_offset of their arenas (keep stats_offset a multiple of 8 so that
- * the rows stay 32-byte aligned).  `block_map` (device int32[total_blocks], may be null) names the
- * tensor of every block; without it each block searches the table.  Results equal a loop of
+ * the rows stay 32-byte aligned).  Results equal a loop of
  * gact_quantize / gact_dequantize over the tensors (gact/gact/quantizer.py:95-142 drives the reference
- * one tensor at a time).  `plan` is the array gact_batch_plan filled.  `dtypes` says which element types
+ * one tensor at a time).  `workspace` is what gact_batch_plan filled for the same table, bits, L and
+ * total_blocks.  `dtypes` says which element types
  * occur in the table, which the host that built it knows: bit 0 float, bit 1 half, bit 2 bfloat16 (GACT_DTYPES_*); quantize
- * launches only the kernels of those types (a half-only kernel needs a third fewer registers than one that
- * also carries the float path), so a tensor whose type is missing from the mask is left unquantized. */
+ * launches only the kernels of those types, so a tensor whose type is missing from the mask is left unquantized. */
 #define GACT_DTYPES_F32 1
 #define GACT_DTYPES_F16 2
 #define GACT_DTYPES_BF16 4
 #define GACT_DTYPES_ALL 7
 int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
-                          int noise_mode, int dtypes, const int64_t* plan, const int32_t* block_map,
-                          void* packed_arena, void* scale_arena, void* min_arena, void* stream);
+                          int noise_mode, int dtypes, const void* workspace, void* packed_arena,
+                          void* scale_arena, void* min_arena, void* stream);
 int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L,
-                            int64_t total_blocks, const int64_t* plan, const int32_t* block_map,
-                            const void* packed_arena, const void* scale_arena, const void* min_arena,
-                            void* stream);
+                            int64_t total_blocks, const void* workspace, const void* packed_arena,
+                            const void* scale_arena, const void* min_arena, void* stream);
 
 #ifdef __cplusplus
 }

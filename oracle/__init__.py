@@ -65,6 +65,7 @@ def lib():
         L.gact_oracle_minimax.argtypes = [vp, i32, i64, i64, vp, vp]
         L.gact_oracle_scale.argtypes = [vp, vp, i32, i32, i64, vp]
         L.gact_oracle_philox4x32_10.argtypes = [vp, vp, vp]
+        L.gact_oracle_philox4x32.argtypes = [vp, vp, i32, vp]
         L.gact_oracle_curand_uniform.argtypes = [ctypes.c_uint32]
         L.gact_oracle_curand_uniform.restype = ctypes.c_float
         L.gact_oracle_noise.argtypes = [i32, u64, i32, i64, i64, i64, vp]
@@ -130,12 +131,19 @@ def scale(mn, mx, bits):
     return out
 
 
-def philox4x32_10(ctr, key):
+def philox4x32(ctr, key, rounds):
     ctr = _c(ctr, np.uint32)
     key = _c(key, np.uint32)
     out = np.empty(4, np.uint32)
-    lib().gact_oracle_philox4x32_10(_p(ctr), _p(key), _p(out))
+    lib().gact_oracle_philox4x32(_p(ctr), _p(key), int(rounds), _p(out))
     return out
+
+
+def philox4x32_10(ctr, key):
+    return philox4x32(ctr, key, 10)
+
+
+FAST_ROUNDS = 7   # Philox rounds of the fast noise stream
 
 
 def curand_uniform(x):

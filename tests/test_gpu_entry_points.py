@@ -268,6 +268,22 @@ def test_batched_refuses_an_arena_that_is_too_small():
     q = bq.quantize(tensors, bits, [0, 1, 2], arena_bytes=1 << 20)
     ok, need = q.ok()
     assert not ok and need == 3 * 4096 * 256
+    # a void launch is an error as soon as its result is used
+    with pytest.raises(RuntimeError, match="void"):
+        q.per_tensor(0)
+    with pytest.raises(RuntimeError, match="void"):
+        bq.dequantize(q)
+
+
+def test_batched_refuses_a_width_it_cannot_pack():
+    # calc_precision started from 32 bits with a loose budget leaves tensors at 32: not a packable width
+    tensors = [torch.randn(512, 256, device="cuda") for _ in range(3)]
+    bq = BatchedQuantizer([t.numel() for t in tensors], [torch.float32] * 3, "cuda")
+    bits = torch.tensor([4, 32, 2], dtype=torch.int32, device="cuda")
+    q = bq.quantize(tensors, bits, [0, 1, 2])
+    assert not q.ok()[0]
+    with pytest.raises(RuntimeError, match="void"):
+        bq.dequantize(q)
 
 
 def test_random_cases_on_general_shapes_masks_and_minimax():

@@ -228,7 +228,7 @@ def test_more_than_2_to_31_elements(bits):
     uu = np.empty(Nt * 256, np.float32)
     cache = {}
     for b in np.unique(blk[:: 8])[:64]:                 # 64 blocks = 512 elements are enough to pin the indexing
-        cache[int(b)] = oracle.philox4x32_10([0, 0, int(b) & 0xFFFFFFFF, int(b) >> 32], [9, 0])
+        cache[int(b)] = oracle.philox4x32([0, 0, int(b) & 0xFFFFFFFF, int(b) >> 32], [9, 0], oracle.FAST_ROUNDS)
     sel = np.nonzero(np.isin(blk, np.array(list(cache), dtype=np.uint64)))[0]
     for e in sel:
         w = int(cache[int(blk[e])][(int(idx[e]) % 8) // 2])

@@ -42,7 +42,7 @@ def test_struct_layout_matches_the_header():
 
 def test_status_codes_and_sizes():
     L = _abi.lib()
-    assert L.gact_abi_version() == 4
+    assert L.gact_abi_version() == 5
     assert L.gact_strerror(0) == b"ok"
     for code in (-1, -2, -3, -4, -5):
         assert L.gact_strerror(code) not in (b"ok", b"unknown error")
@@ -70,8 +70,14 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     assert L.gact_unpack(16, 5, 16, 16, 0, 4, 1, 256, 16, None) == -1
     assert L.gact_mask_pack(None, -1, None, None) == -1
     assert L.gact_calc_precision_device(16, 16, 16, 5000, 1.0, None, None) == -3                 # beyond the LDS table
-    assert L.gact_quantize_batched(16, 16, 3, 3, 1, 3, 16, None, 16, 16, 16, None) == -1         # injected noise
-    assert L.gact_quantize_batched(16, 16, 3, 3, 0, 8, 16, None, 16, 16, 16, None) == -1         # dtype mask
+    assert L.gact_quantize_batched(16, 16, 3, 3, 1, 3, 16, 16, 16, 16, None) == -1               # injected noise
+    assert L.gact_quantize_batched(16, 16, 3, 3, 0, 8, 16, 16, 16, 16, None) == -1               # dtype mask
+    assert L.gact_quantize_batched(16, 16, 3, 3, 0, 3, 8, 16, 16, 16, None) == -2                # misaligned workspace
+    assert L.gact_batch_plan(16, 16, 3, 3, -1, 16, None) == -1                                   # negative capacity
+    assert L.gact_batch_plan(16, 16, 3, 3, 100, None, None) == -1                                # no workspace
+    # header (32 int64) + one int32 per tensor, padded to 64 + one int32 per block, padded to 2 + 8 bytes per block
+    assert L.gact_batch_workspace_bytes(3, 5) == 256 + 64 * 4 + 6 * 4 + 5 * 8
+    assert L.gact_batch_workspace_bytes(-1, 5) == -1
     assert L.gact_quantize(16, 3, 256, 4, 0, 0, None, 16, 16, 16, None, None) == -1               # element type
     assert L.gact_quantize(0, 2, 256, 4, 0, 0, None, 16, 16, 16, None, None) == -1                # bfloat16, null data
     assert L.gact_minimax(16, 2, 4, 64, 16, 16, None) == -1                                      # no bfloat16 here

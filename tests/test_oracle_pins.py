@@ -111,6 +111,16 @@ def test_philox_known_answers():
     ]
     for ctr, key, want in kat:
         assert [int(v) for v in oracle.philox4x32_10(ctr, key)] == want
+    # and for philox4x32 with 7 rounds (the fast stream's generator), same file
+    kat7 = [
+        ([0, 0, 0, 0], [0, 0], [0x5f6fb709, 0x0d893f64, 0x4f121f81, 0x4f730a48]),
+        ([0xffffffff] * 4, [0xffffffff] * 2, [0x5207ddc2, 0x45165e59, 0x4d8ee751, 0x8c52f662]),
+        ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0],
+         [0x4dfccaba, 0x190a87f0, 0xc47362ba, 0xb6b5242a]),
+    ]
+    for ctr, key, want in kat7:
+        assert [int(v) for v in oracle.philox4x32(ctr, key, 7)] == want
+    assert oracle.FAST_ROUNDS == 7
 
 
 def test_curand_uniform_map_closed_form():
@@ -143,7 +153,7 @@ def test_fast_stream_definition():
     seed = 7
     u = oracle.noise(oracle.NOISE_FAST, seed, 4, 3).reshape(-1)
     for E in (0, 1, 7, 8, 300, 767):
-        blk = oracle.philox4x32_10([0, 0, E // 8, 0], [seed, 0])
+        blk = oracle.philox4x32([0, 0, E // 8, 0], [seed, 0], oracle.FAST_ROUNDS)
         w = int(blk[(E % 8) // 2])
         h = (w >> 16) if (E % 2) else (w & 0xFFFF)
         assert u[E] == np.float32((h + 0.5) / 65536.0)
