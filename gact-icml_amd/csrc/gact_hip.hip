@@ -29,6 +29,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
 #include <queue>
 #include <type_traits>
 #include <utility>
@@ -2131,6 +2132,7 @@ const char* gact_strerror(int code) {
     case GACT_ESHAPE: return "unsupported shape";
     case GACT_ELAUNCH: return "HIP launch failed";
     case GACT_EBUDGET: return "bit budget unreachable: every tensor is already at 1 bit";
+    case GACT_ELIMIT: return "beyond the limit of the library's own workspace (4096 tensors, 262144 blocks of 128 groups)";
   }
   return "unknown error";
 }
@@ -2412,6 +2414,59 @@ int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, 
                      batch_workspace(const_cast<void*>(workspace), L, total_blocks), (const uint8_t*)packed_arena,
                      (const uint8_t*)scale_arena, (const uint8_t*)min_arena);
   return launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// The batched quantize for callers that cannot allocate: plan + quantize with the workspace in a device array
+// of the library's own.  Every GPU the library runs on holds its own copy of the array, at its own address,
+// until the process ends; the address is looked up once per device (the array's name is only a host-side
+// handle) and that pointer is what the kernels get.  Calls on one GPU share the array: they must not overlap.
+// Nothing in it has to start at zero - the plan kernels write every field the work kernels read.
+// ------------------------------------------------------------------------------------------------
+#define GACT_STATIC_MAX_TENSORS 4096
+#define GACT_STATIC_MAX_BLOCKS 262144
+#define GACT_STATIC_WORKSPACE_BYTES (256 + GACT_STATIC_MAX_TENSORS * 4 + GACT_STATIC_MAX_BLOCKS * 12)
+#define GACT_MAX_DEVICES 64
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[GACT_STATIC_WORKSPACE_BYTES];
+
+namespace {
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[GACT_MAX_DEVICES];  // device address of `scratch` on each device, once looked up
+
+int static_workspace(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= GACT_MAX_DEVICES) return GACT_ELAUNCH;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return GACT_ELAUNCH;
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return GACT_OK;
+}
+}  // namespace
+
+int gact_quantize_batched_static(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
+                                 int64_t capacity, int noise_mode, int dtypes, void* packed_arena, void* scale_arena,
+                                 void* min_arena, void* stream) {
+  if (!batched_args_ok(L, total_blocks) || capacity < 0) return GACT_EINVAL;
+  if (noise_mode != GACT_NOISE_CONST && noise_mode != GACT_NOISE_REF && noise_mode != GACT_NOISE_FAST) return GACT_EINVAL;
+  if (dtypes < 0 || dtypes > GACT_DTYPES_ALL) return GACT_EINVAL;
+  if (dtypes == 0) dtypes = GACT_DTYPES_ALL;
+  if (L > GACT_STATIC_MAX_TENSORS || total_blocks > GACT_STATIC_MAX_BLOCKS) return GACT_ELIMIT;
+  static_assert(GACT_STATIC_WORKSPACE_BYTES >= 256 + GACT_STATIC_MAX_TENSORS * 4 + GACT_STATIC_MAX_BLOCKS * 4 + GACT_STATIC_MAX_BLOCKS * 8,
+                "the array holds the workspace of the largest table");
+  if (L == 0 || total_blocks == 0) return GACT_OK;
+  if (!table || !bits || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
+  if (!aligned16(packed_arena)) return GACT_EALIGN;
+  void* ws = nullptr;
+  const int rc = static_workspace(&ws);
+  if (rc != GACT_OK) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const int planned = batch_plan_on(table, bits, L, total_blocks, capacity, ws, s);
+  if (planned != GACT_OK) return planned;
+  return quantize_batched_on(table, L, total_blocks, noise_mode, dtypes, ws, packed_arena, scale_arena, min_arena, s);
 }
 
 }  // extern "C"

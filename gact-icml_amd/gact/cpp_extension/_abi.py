@@ -54,6 +54,7 @@ SIGNATURES = {
     "gact_batch_plan": (_i32, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
     "gact_quantize_batched": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "gact_dequantize_batched": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "gact_quantize_batched_static": (_i32, [_vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp]),
 }
 
 

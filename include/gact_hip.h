@@ -41,6 +41,7 @@ extern "C" {
 #define GACT_ESHAPE (-3) /* shape not supported by this entry point                               */
 #define GACT_ELAUNCH (-4) /* the HIP runtime reported an error at launch                          */
 #define GACT_EBUDGET (-5) /* calc_precision: every tensor is at 1 bit and the budget is not met   */
+#define GACT_ELIMIT (-6)  /* beyond the size limit of an entry point that brings its own workspace */
 
 const char* gact_strerror(int code);
 int gact_abi_version(void);
@@ -151,6 +152,20 @@ int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, in
 int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L,
                             int64_t total_blocks, const void* workspace, const void* packed_arena,
                             const void* scale_arena, const void* min_arena, void* stream);
+
+/* gact_batch_plan followed by gact_quantize_batched, with the workspace in a device array that is part of
+ * the library (about 3.2 MB per GPU the library runs on, held until the process ends) instead of memory the
+ * caller brings: nothing is allocated, by the library or on its behalf.  No counterpart in the reference; it
+ * is for callers that cannot allocate - code under HIP graph capture, tight serving loops, harnesses that
+ * forbid it.  Same results as the two calls it stands for (packed_offset of every table entry is filled, the
+ * arenas are written); the plan's verdict stays in the library's array, so size the arena for the worst case
+ * or check the widths beforehand.  Limits: L <= 4096 tensors and total_blocks <= 262144 (33.5 M groups),
+ * GACT_ELIMIT beyond.  All calls on one GPU share the array: calls that overlap on one GPU (two streams, two
+ * threads) race, the caller serialises them.  The first call on a GPU looks the array's address up; make it
+ * outside a stream capture.  Dequantize with gact_batch_plan + gact_dequantize_batched as usual. */
+int gact_quantize_batched_static(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
+                                 int64_t capacity, int noise_mode, int dtypes, void* packed_arena,
+                                 void* scale_arena, void* min_arena, void* stream);
 
 #ifdef __cplusplus
 }
