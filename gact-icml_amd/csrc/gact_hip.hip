@@ -569,41 +569,49 @@ __device__ __forceinline__ uint32_t swap_with_neighbour(uint32_t v) {
   return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0xB1, 0xf, 0xf, false);
 }
 
-// The fast stream's uniforms for all chunks of group n that lane i owns.  One Philox block feeds 8
-// consecutive elements.  With 8-column chunks that is one block per chunk; with 4-column chunks two
-// neighbouring lanes share a block, so the even lane computes the block of chunk m, the odd lane the
-// block of chunk m+1, and they exchange the halves the other one needs.
+// The fast stream.  A group of 256 elements draws 16 Philox blocks; block j serves columns 8j .. 8j+7 with its
+// eight 16-bit pieces h (word by word, low half first): u = (h + 0.5) * 2^-16.  The column 128 further on
+// takes 1 - u, the same draw mirrored: every element's noise is uniform on the same grid, and the two elements of
+// a pair (which sit half a group apart) round in opposite directions more often than not (their rounding errors
+// have covariance <= 0).  Half the Philox work, and no second conversion for the mirrored half.
+// In terms of the flat element index E: block (E / 256) * 16 + (E % 128) / 8, piece E % 8, mirrored if E % 256 >= 128.
+__device__ __forceinline__ uint64_t fast_block_of(uint64_t E) { return (E >> 8) * 16 + ((E & 127) >> 3); }
+__device__ __forceinline__ float fast_mirror(float u) { return 1.0f - u; }   // exact: u has 17 significant bits
+
+// The fast stream's uniforms for all chunks of group n that lane i owns.  With 8-column chunks (8i + 128m) the
+// lane's two chunks are one block and its mirror image.  With 4-column chunks (4i + 64m) chunks 0 and 1 are halves
+// of blocks i/2 and 8 + i/2, which two neighbouring lanes share: the even lane computes the first, the odd lane the
+// second, and they exchange the halves the other one needs; chunks 2 and 3 are the mirror images of 0 and 1.
 template <typename T>
 __device__ __forceinline__ void fast_noise(int64_t n, int i, uint32_t k0, uint32_t k1,
                                            float (&u)[Elem<T>::kQChunks][Elem<T>::kQWidth]) {
   constexpr int CH = Elem<T>::kQChunks, W = Elem<T>::kQWidth;
+  uint32_t r[4];
   if (W == 8) {
+    static_assert(W != 8 || CH == 2, "two chunks of 8 columns, 128 apart");
+    const uint64_t blk = (uint64_t)n * 16 + i;
+    philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
 #pragma unroll
-    for (int k = 0; k < CH; k++) {
-      const uint64_t blk = (uint64_t)n * (GROUP / 8) + 16 * k + i;
-      uint32_t r[4];
-      philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
-#pragma unroll
-      for (int e = 0; e < W; e++) u[k][e] = fast_piece(r[(e >> 2) * 2], r[(e >> 2) * 2 + 1], e & 3);
+    for (int e = 0; e < W; e++) {
+      u[0][e] = fast_piece(r[(e >> 2) * 2], r[(e >> 2) * 2 + 1], e & 3);
+      u[CH - 1][e] = fast_mirror(u[0][e]);
     }
   } else {
+    static_assert(W == 8 || CH == 4, "four chunks of 4 columns, 64 apart");
     const bool odd = i & 1;
+    const uint64_t blk = (uint64_t)n * 16 + (odd ? 8 : 0) + (i >> 1);
+    philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
+    // the even lane owns elements 0..3 of a block (words 0,1), the odd lane elements 4..7 (words 2,3)
+    const uint32_t ga = swap_with_neighbour(odd ? r[0] : r[2]);
+    const uint32_t gb = swap_with_neighbour(odd ? r[1] : r[3]);
+    const uint32_t a0 = odd ? ga : r[0], a1 = odd ? gb : r[1];   // chunk 0: block i/2
+    const uint32_t b0 = odd ? r[2] : ga, b1 = odd ? r[3] : gb;   // chunk 1: block 8 + i/2
 #pragma unroll
-    for (int m = 0; m < CH; m += 2) {
-      // element block of (chunk, lane): (4*(16*chunk + lane)) / 8 = 8*chunk + lane/2
-      const uint64_t blk = (uint64_t)n * (GROUP / 8) + 8 * (m + (odd ? 1 : 0)) + (i >> 1);
-      uint32_t r[4];
-      philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
-      // the even lane owns elements 0..3 of a block (words 0,1), the odd lane elements 4..7 (words 2,3)
-      const uint32_t ga = swap_with_neighbour(odd ? r[0] : r[2]);
-      const uint32_t gb = swap_with_neighbour(odd ? r[1] : r[3]);
-      const uint32_t a0 = odd ? ga : r[0], a1 = odd ? gb : r[1];   // chunk m
-      const uint32_t b0 = odd ? r[2] : ga, b1 = odd ? r[3] : gb;   // chunk m + 1
-#pragma unroll
-      for (int e = 0; e < W; e++) {
-        u[m][e] = fast_piece(a0, a1, e);
-        u[m + 1][e] = fast_piece(b0, b1, e);
-      }
+    for (int e = 0; e < W; e++) {
+      u[0][e] = fast_piece(a0, a1, e);
+      u[1 % CH][e] = fast_piece(b0, b1, e);
+      u[2 % CH][e] = fast_mirror(u[0][e]);
+      u[3 % CH][e] = fast_mirror(u[1 % CH][e]);
     }
   }
 }
@@ -1092,17 +1100,25 @@ __device__ __forceinline__ void quantize_supergroup_wide(const T* __restrict__ x
     for (int g = 0; g < WPT; g += STEP) {
       float u[STEP][W];
       if (NOISE == GACT_NOISE_FAST) {
+        // lane l owns columns W*l ..: the lanes of the upper half of the group take the mirror image of what the
+        // lanes of the lower half draw, so both halves compute the same block
+        constexpr int HALF = LPS / 2;
+        const int lh = l & (HALF - 1);
+        const bool upper = l >= HALF;
         if (W == 8) {
-          const uint64_t blk = (uint64_t)(n0 + g) * (GROUP / 8) + l;
+          const uint64_t blk = (uint64_t)(n0 + g) * 16 + lh;
           uint32_t r[4];
           philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
 #pragma unroll
-          for (int e = 0; e < W; e++) u[0][e] = fast_piece(r[(e >> 2) * 2], r[(e >> 2) * 2 + 1], e & 3);
+          for (int e = 0; e < W; e++) {
+            const float d = fast_piece(r[(e >> 2) * 2], r[(e >> 2) * 2 + 1], e & 3);
+            u[0][e] = upper ? fast_mirror(d) : d;
+          }
         } else {
-          // a Philox block feeds 8 consecutive elements = the columns of a pair of neighbouring lanes: the even
+          // a Philox block feeds 8 consecutive columns = those of a pair of neighbouring lanes: the even
           // lane computes the block of group g, the odd lane that of group g + 1, and they exchange halves
           const bool odd = l & 1;
-          const uint64_t blk = (uint64_t)(n0 + g + (odd ? 1 : 0)) * (GROUP / 8) + (l >> 1);
+          const uint64_t blk = (uint64_t)(n0 + g + (odd ? 1 : 0)) * 16 + (lh >> 1);
           uint32_t r[4];
           philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
           const uint32_t ga = swap_with_neighbour(odd ? r[0] : r[2]);
@@ -1111,8 +1127,9 @@ __device__ __forceinline__ void quantize_supergroup_wide(const T* __restrict__ x
           const uint32_t b0 = odd ? r[2] : ga, b1 = odd ? r[3] : gb;   // group g + 1
 #pragma unroll
           for (int e = 0; e < W; e++) {
-            u[0][e] = fast_piece(a0, a1, e);
-            u[STEP - 1][e] = fast_piece(b0, b1, e);
+            const float da = fast_piece(a0, a1, e), db = fast_piece(b0, b1, e);
+            u[0][e] = upper ? fast_mirror(da) : da;
+            u[STEP - 1][e] = upper ? fast_mirror(db) : db;
           }
         }
       } else {
@@ -1285,10 +1302,11 @@ pack_any_kernel(const T* __restrict__ data, const T* __restrict__ mn, const T* _
       if ((ni & 3) == 0) philox4x32<PHILOX_REF_ROUNDS>(ni >> 2, 0u, (uint32_t)j, (uint32_t)((uint64_t)j >> 32), k0, k1, r);
       u = curand_uniform_map(r[ni & 3]);
     } else if (NOISE == GACT_NOISE_FAST) {
-      const uint64_t blk = (uint64_t)id >> 3;
+      const uint64_t blk = fast_block_of((uint64_t)id);
       philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
       const int e = (int)(id & 7);
       u = fast_uniform_map((e & 1) ? (r[e >> 1] >> 16) : (r[e >> 1] & 0xffffu));
+      if (id & 128) u = fast_mirror(u);
     }
     typename Elem<T>::Store one;
     Elem<T>::set(one, 0, 0, data[id]);
@@ -1354,10 +1372,13 @@ pack_rows8_kernel(const T* __restrict__ data, const T* __restrict__ mn, const T*
         u[e] = curand_uniform_map(r[e][ni & 3]);
       }
     } else if (NOISE == GACT_NOISE_FAST) {
-      const uint64_t blk = (uint64_t)id0 >> 3;
+      const uint64_t blk = fast_block_of((uint64_t)id0);
       philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r[0]);
 #pragma unroll
-      for (int e = 0; e < 8; e++) u[e] = fast_uniform_map((e & 1) ? (r[0][e >> 1] >> 16) : (r[0][e >> 1] & 0xffffu));
+      for (int e = 0; e < 8; e++) {
+        u[e] = fast_uniform_map((e & 1) ? (r[0][e >> 1] >> 16) : (r[0][e >> 1] & 0xffffu));
+        if (id0 & 128) u[e] = fast_mirror(u[e]);
+      }
     } else {
 #pragma unroll
       for (int e = 0; e < 8; e++) u[e] = 0.5f;

@@ -115,8 +115,13 @@ def dequantize_and_unpack(data, shape, q_bit, scale, mn):
 
 
 def op_quantize_mask(input):
-    """gact/gact/ops.py:49-50."""
-    return [ext_quantization.act_quantize_dropout_mask(input.contiguous()), input.shape]
+    """gact/gact/ops.py:49-50.  The mask kernel reads 16 bytes per lane: a contiguous view that starts at
+    an odd storage offset (a slice, a chunk) is copied to a fresh allocation first, as the float path does
+    (the reference's kernel takes any alignment)."""
+    data = input.contiguous()
+    if not _abi.aligned(data):
+        data = data.clone()
+    return [ext_quantization.act_quantize_dropout_mask(data), input.shape]
 
 
 def op_dequantize_mask(input):

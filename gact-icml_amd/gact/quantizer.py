@@ -22,6 +22,7 @@ class _Swap:
     def __init__(self, prefetch):
         self.out_stream = torch.cuda.Stream()
         self.in_stream = torch.cuda.Stream()
+        self.prefetch_started = self.prefetch_done = None
         if prefetch:
             self.prefetch_started = torch.cuda.Event(blocking=True)
             self.prefetch_done = torch.cuda.Event(blocking=True)
@@ -34,7 +35,9 @@ class Quantizer:
     def __init__(self, default_bit, swap, prefetch):
         self.default_bit = default_bit
         self.swap, self.prefetch = swap, prefetch
-        self._swap = _Swap(prefetch) if swap else None
+        # the reference creates the prefetch events whenever prefetch is set, with or without swap
+        # (quantizer.py:25-28): start_prefetch_event / end_prefetch_event exist in both cases
+        self._swap = _Swap(prefetch) if (swap or prefetch) else None
         self.compute_stream = torch.cuda.current_stream() if torch.cuda.is_available() else None
 
         self.unrelated_tensors = set()   # data pointers of parameters: saved for backward, never compressed
@@ -90,8 +93,8 @@ class Quantizer:
         if t.data_ptr() in self.unrelated_tensors:
             return False, False
         if t.dtype == torch.uint8 and t.numel() > 0:
-            lo, hi = torch.aminmax(t)                 # one reduction and one synchronisation for both ends
-            is_mask = (int(lo), int(hi)) == (0, 1)
+            # one reduction and one synchronisation for both ends
+            is_mask = torch.stack(torch.aminmax(t)).tolist() == [0, 1]
             return is_mask, is_mask
         if t.dtype == torch.bool:
             # contiguous only: an expanded or strided view (a broadcast attention mask) may occupy far less than
@@ -100,6 +103,8 @@ class Quantizer:
                        and t.is_contiguous())
             return is_mask, is_mask
         ok = t.dtype in _COMPRESSIBLE and t.requires_grad is not False and t.dim() in _RANKS
+        if ok and t.dtype == torch.bfloat16 and config.group_size != 256:
+            ok = False      # bfloat16 exists in the single-pass kernels (group size 256) only: left alone, as in the reference
         return ok, False
 
     def generate_tensor_key(self, t, tid):

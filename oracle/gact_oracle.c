@@ -243,27 +243,32 @@ static inline float ref_stream_uniform(uint64_t seed, uint64_t byte_index, int d
   return gact_oracle_curand_uniform(out[draw & 3]);
 }
 
-/* The fast noise stream (ours; the reference has no counterpart).  One       */
-/* Philox4x32-7 block (the same round function, seven rounds: the fewest for */
-/* which Random123's authors report that the generator passes BigCrush; its  */
-/* kat_vectors hold the 7-round known answers too) serves 8 consecutive      */
-/* elements of the flattened tensor:                                         */
-/* key = seed, counter = (0, 0, E/8 lo, E/8 hi); element E takes 16 bits:     */
-/* word (E%8)/2, low half first; u = (h + 0.5) * 2^-16, which lies strictly   */
-/* inside (0, 1) and is symmetric about 1/2.                                  */
+/* The fast noise stream (ours; the reference has no counterpart).  Philox4x32 */
+/* with seven rounds (the same round function; the fewest rounds for which    */
+/* Random123's authors report that the generator passes BigCrush; its         */
+/* kat_vectors hold the 7-round known answers too), key = seed.  Every 256    */
+/* consecutive elements of the flattened tensor draw 16 blocks: element E     */
+/* takes block (E/256)*16 + (E%128)/8 (counter = (0, 0, block lo, block hi)),  */
+/* of it the 16-bit piece E%8 (word (E%8)/2, low half first), h;               */
+/* u = (h + 0.5) * 2^-16 for E%256 < 128 and 1 - that for E%256 >= 128: the    */
+/* two elements half a group apart share one draw, mirrored (an antithetic     */
+/* pair: both uniform on the same grid, strictly inside (0, 1), symmetric      */
+/* about 1/2; covariance of their rounding errors <= 0).                       */
 #define GACT_FAST_ROUNDS 7
 static inline float fast_stream_uniform_from_block(const uint32_t out[4], int e8) {
   uint32_t w = out[e8 >> 1];
   uint32_t h = (e8 & 1) ? (w >> 16) : (w & 0xffffu);
   return (float)(2u * h + 1u) * 7.62939453125e-06f; /* (2h+1) * 2^-17, exact */
 }
+static inline uint64_t fast_stream_block(uint64_t elem) { return (elem >> 8) * 16u + ((elem & 127u) >> 3); }
 static inline float fast_stream_uniform(uint64_t seed, uint64_t elem) {
-  uint64_t blk = elem >> 3;
+  uint64_t blk = fast_stream_block(elem);
   uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
   uint32_t ctr[4] = {0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32)};
   uint32_t out[4];
   gact_oracle_philox4x32(ctr, key, GACT_FAST_ROUNDS, out);
-  return fast_stream_uniform_from_block(out, (int)(elem & 7));
+  float u = fast_stream_uniform_from_block(out, (int)(elem & 7));
+  return (elem & 128u) ? 1.0f - u : u; /* exact: 17 significant bits */
 }
 
 #define GACT_NOISE_CONST 0  /* u = 0.5 for every element: deterministic rounding */

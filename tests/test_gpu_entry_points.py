@@ -102,6 +102,30 @@ def test_pack_with_min_max_narrower_than_the_data(dtype, bits, ngd):
         np.testing.assert_array_equal(bits_view(out.cpu().numpy().reshape(-1)), bits_view(ref.reshape(-1)))
 
 
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("ngd", [(67, 1, 256), (13, 2, 96), (21, 1, 128)])
+def test_pack_codes_past_two_to_the_31_saturate_like_the_signed_conversion(bits, ngd):
+    """float32 with caller-supplied min = max = 0: scale = (2^bits - 1) / 2e-6, so data up to 1e5 gives codes from 0
+    to beyond 2^33.  The reference converts with __float2int_rn, which saturates at 0x7fffffff: from 2^31 on the
+    low byte of a code is 0xff, not the low byte of the value (quantization_cuda_kernel.cu:66-67).  Every
+    kernel behind gact_pack (the row kernel at D = 256, 8 columns per thread, one thread per byte)."""
+    N, G, D = ngd
+    g = torch.Generator().manual_seed(7 + bits)
+    mag = torch.pow(10.0, torch.rand((N, G, D), generator=g) * 8.0 - 3.0)       # 1e-3 .. 1e5
+    x = (mag * (torch.rand((N, G, D), generator=g) < 0.9)).to(torch.float32)   # some exact zeros, no negatives needed
+    x[0, 0, :8] = torch.tensor([4294.9673, 4294.9674, 2147.4836, 2147.4837, 1073.7418, 1073.7419, 8589.9346, 0.0])
+    mn_np = np.zeros(N * G, np.float32)
+    sc_np = oracle.scale(mn_np, mn_np, bits)
+    top = float(x.max()) * float(sc_np[0])
+    assert top > 2.0 ** 33 and sc_np[0] == np.float32((2 ** bits - 1) / 2e-6)
+    mn = torch.zeros((N, G, 1), device="cuda")
+    for stream, mode in (("deterministic", 0), ("reference", 2), ("fast", 3)):
+        want = oracle.pack(x.numpy(), mn_np, sc_np, bits, mode, 5)
+        packed, scale = ext_quantization.pack_single_precision(x.cuda(), mn, mn.clone(), bits, True, 5, rng_stream=stream)
+        np.testing.assert_array_equal(bits_view(scale.cpu().numpy().reshape(-1)), bits_view(sc_np))
+        np.testing.assert_array_equal(packed.cpu().numpy().view(np.uint8)[:want.size], want, err_msg=stream)
+
+
 def test_pack_uses_the_min_max_it_is_given():
     # the entry point's contract: codes are taken against the caller's min / max, whatever the data holds
     x = torch.rand((16, 1, 256)) * 0.5 + 0.25
@@ -123,6 +147,18 @@ def test_dropout_mask(n):
     np.testing.assert_array_equal(q[0].cpu().numpy(), oracle.mask_pack(data.numpy()))
     out = ops.op_dequantize_mask(q)
     assert out.dtype == torch.uint8 and torch.equal(out.cpu(), data)
+
+
+def test_dropout_mask_views_that_start_at_an_odd_offset():
+    # a contiguous slice or chunk of a mask starts where it starts: the reference's kernel takes any alignment
+    g = torch.Generator().manual_seed(9)
+    whole = (torch.rand(5000, generator=g) < 0.4).to(torch.uint8).cuda()
+    for view in (whole[1:], whole[3:4100], whole.view(50, 100)[7:], whole.view(torch.bool)[5:]):
+        assert view.is_contiguous() and view.data_ptr() % 16 != 0
+        data = view.view(torch.uint8) if view.dtype == torch.bool else view
+        q = ops.op_quantize_mask(data)
+        np.testing.assert_array_equal(q[0].cpu().numpy(), oracle.mask_pack(data.cpu().numpy().reshape(-1)))
+        assert torch.equal(ops.op_dequantize_mask(q), data)
 
 
 def test_dropout_mask_every_count_of_blocks_a_wave_can_end_on():

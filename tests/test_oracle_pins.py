@@ -149,15 +149,47 @@ def test_reference_stream_walks_the_counter_like_curand():
     assert u2[2, 0, 1] == np.float32(oracle.curand_uniform(int(blk[2])))
 
 
+def fast_stream_expected(seed, E):
+    """The fast stream restated from its definition: block (E/256)*16 + (E%128)/8 of Philox4x32-7, piece E%8,
+    u = (h + 0.5) / 2^16, mirrored (1 - u) in the upper half of every 256."""
+    blk = (E // 256) * 16 + (E % 128) // 8
+    out = oracle.philox4x32([0, 0, blk & 0xFFFFFFFF, blk >> 32], [seed & 0xFFFFFFFF, seed >> 32], oracle.FAST_ROUNDS)
+    w = int(out[(E % 8) // 2])
+    h = (w >> 16) if (E % 2) else (w & 0xFFFF)
+    u = Fraction(2 * h + 1, 1 << 17)
+    return float(1 - u if E % 256 >= 128 else u)
+
+
 def test_fast_stream_definition():
     seed = 7
     u = oracle.noise(oracle.NOISE_FAST, seed, 4, 3).reshape(-1)
-    for E in (0, 1, 7, 8, 300, 767):
-        blk = oracle.philox4x32([0, 0, E // 8, 0], [seed, 0], oracle.FAST_ROUNDS)
-        w = int(blk[(E % 8) // 2])
-        h = (w >> 16) if (E % 2) else (w & 0xFFFF)
-        assert u[E] == np.float32((h + 0.5) / 65536.0)
+    for E in (0, 1, 7, 8, 127, 128, 129, 135, 255, 256, 300, 383, 384, 500, 767):
+        assert u[E] == np.float32(fast_stream_expected(seed, E)), E
     assert 0.0 < u.min() and u.max() < 1.0
+    # the two halves of every 256 are mirror images, and every value sits on the (k + 0.5) / 2^16 grid
+    g = u.reshape(3, 2, 128)
+    assert np.array_equal(g[:, 1, :], np.float32(1.0) - g[:, 0, :])
+    k = u.astype(np.float64) * 65536.0 - 0.5
+    assert np.array_equal(k, np.round(k)) and k.min() >= 0 and k.max() <= 65535
+
+
+def test_fast_stream_marginals_and_pair_covariance():
+    """Each element's noise is uniform on the grid; the mirrored pair makes the rounding errors of the two
+    elements negatively correlated, never positively: cov(up_i, up_j) = max(0, f_i + f_j - 1) - f_i f_j <= 0."""
+    u = oracle.noise(oracle.NOISE_FAST, 11, 8, 4096).reshape(-1, 256).astype(np.float64)   # 4096 groups
+    assert abs(u.mean() - 0.5) < 2e-3 and abs(u.var() - 1.0 / 12.0) < 2e-3
+    lower, upper = u[:, :128], u[:, 128:]
+    assert abs(lower.mean() - 0.5) < 2e-3 and abs(upper.mean() - 0.5) < 2e-3
+    for fi, fj in ((0.3, 0.3), (0.7, 0.6), (0.5, 0.5), (0.9, 0.2)):
+        up_i = lower >= 1.0 - fi
+        up_j = upper >= 1.0 - fj
+        assert abs(up_i.mean() - fi) < 5e-3 and abs(up_j.mean() - fj) < 5e-3
+        cov = (up_i & up_j).mean() - up_i.mean() * up_j.mean()
+        want = max(0.0, fi + fj - 1.0) - fi * fj
+        assert abs(cov - want) < 5e-3 and cov < 1e-3
+    # neighbours inside a block, and elements of different blocks, are uncorrelated
+    for a, b in ((u[:, 0], u[:, 1]), (u[:, 5], u[:, 77]), (u[:-1, 9], u[1:, 9])):
+        assert abs(np.corrcoef(a, b)[0, 1]) < 0.05
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])

@@ -52,6 +52,13 @@ def test_filter_rules(rec):
     assert q.check_quantize(torch.tensor([0, 2, 1, 0], dtype=torch.uint8)) == (False, False)
     assert q.check_quantize(torch.zeros(4, dtype=torch.uint8)) == (False, False)
     assert q.check_quantize(torch.ones(8192, dtype=torch.bool)) == (False, False)   # bool masks: only on the GPU
+    # bfloat16 (not in the reference) exists in the group-256 kernels only; with another group size it is left alone
+    bf = torch.randn(4, 4).bfloat16().requires_grad_()
+    assert q.check_quantize(bf) == (True, False)
+    config.group_size = 128
+    assert q.check_quantize(bf) == (False, False)
+    assert q.check_quantize(act((4, 4))) == (True, False)
+    config.group_size = 256
 
 
 def test_tuple_protocol_tids_seeds_and_tables(rec):
