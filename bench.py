@@ -211,6 +211,16 @@ def run_ceilings(torch, timer):
     for name, fn, moved in (("device_copy", copy, 2 * nbytes), ("fill", fill, nbytes), ("read_minimax", read, nbytes + 8 * N)):
         ms, _ = timer(fn)
         out[name] = {"us": ms * 1e3, "gbs": moved / (ms * 1e-3) / 1e9, "frac": moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    # what a launch costs whatever it moves: one group of 256 elements through the same entry point, replayed the same way
+    tiny, tq = x.reshape(-1)[:256], torch.empty((65,), dtype=torch.int8, device="cuda")
+    ts, tm = torch.empty((1,), dtype=x.dtype, device="cuda"), torch.empty((1,), dtype=x.dtype, device="cuda")
+
+    def one_group(k):
+        _abi.check(lib.gact_quantize(tiny.data_ptr(), _abi.F32, 256, 2, _abi.NOISE_CONST, 0, None, tq.data_ptr(),
+                                     ts.data_ptr(), tm.data_ptr(), None, torch.cuda.current_stream().cuda_stream))
+
+    ms, _ = timer(one_group)
+    out["launch_floor_us"] = ms * 1e3
     return out
 
 

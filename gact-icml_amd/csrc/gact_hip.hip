@@ -7,10 +7,9 @@
 // 8i + 128m - so every load instruction of a row reads 256 contiguous bytes.  Per-group reductions are
 // four row_ror DPP steps that never leave the row, and - because the reference packs the SAME column of
 // 8/bits consecutive groups into one byte - the lane that owns a column owns every code of that byte:
-// packing needs no cross-lane traffic at all.  One Philox block feeds 8 consecutive elements: a half
-// chunk, or the two float chunks of a pair of neighbouring lanes (which swap the halves they need).
-// Float and bfloat16 at 1 bit, whose rows would hold 8 groups in registers, spread a super-group over a
-// whole wave / half a wave instead (quantize_supergroup_wide): one chunk per lane and group.
+// packing needs no cross-lane traffic at all.  One Philox block feeds 8 consecutive columns - a half
+// chunk, or the float chunks of a pair of neighbouring lanes (which swap the halves they need) - and, mirrored,
+// the 8 columns half a group further on, which the same lane owns.
 //
 // Dequantize has no reduction, so a unit of 8 consecutive groups goes to a whole wave (float: lane l owns
 // columns 4l .. 4l+3) or half a wave (half: 8l .. 8l+7): one 16-byte store per lane and group, every store
@@ -69,46 +68,6 @@ __device__ __forceinline__ void row_all_minmax(float& lo, float& hi) {
 __device__ __forceinline__ void row_all_minmax(f16& lo, f16& hi) {
   asm(GACT_DPP_ALL("v_min_f16_dpp", "v_max_f16_dpp") : "+v"(lo), "+v"(hi));
 }
-// min / max across the 2 or 4 rows of a group of LANES lanes (32 or 64), after the row reduction: exchanges
-// with the lane 16 (and 32) away; every lane of the group ends with the result
-__device__ __forceinline__ float lane_xor(float v, int m) { return __shfl_xor(v, m, 64); }
-__device__ __forceinline__ f16 lane_xor(f16 v, int m) {
-  return __builtin_bit_cast(f16, (uint16_t)__shfl_xor((int)__builtin_bit_cast(uint16_t, v), m, 64));
-}
-// neither operand is NaN here (see row_all_minmax), so the bare instruction will do: the compiler's minnum /
-// maxnum put a canonicalising v_max v, v, v in front of every operand
-__device__ __forceinline__ float min_of(float a, float b) {
-  float r;
-  asm("v_min_f32_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
-}
-__device__ __forceinline__ float max_of(float a, float b) {
-  float r;
-  asm("v_max_f32_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
-}
-__device__ __forceinline__ f16 min_of(f16 a, f16 b) {
-  f16 r;
-  asm("v_min_f16_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
-}
-__device__ __forceinline__ f16 max_of(f16 a, f16 b) {
-  f16 r;
-  asm("v_max_f16_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
-}
-template <int LANES, typename S>
-__device__ __forceinline__ void rows_all_minmax(S& lo, S& hi) {
-  if (LANES >= 32) {
-    lo = min_of(lo, lane_xor(lo, 16));
-    hi = max_of(hi, lane_xor(hi, 16));
-  }
-  if (LANES >= 64) {
-    lo = min_of(lo, lane_xor(lo, 32));
-    hi = max_of(hi, lane_xor(hi, 32));
-  }
-}
-
 // ------------------------------------------------------------------------------------------------
 // Philox4x32.  The key schedule only depends on the seed, so it stays on the scalar unit; each
 // round is two 32x32->64 multiplies and two three-input XORs (v_bitop3_b32, truth table 0x96).
@@ -240,19 +199,16 @@ template <> struct Elem<float> {
   __device__ static __forceinline__ float init_hi() { return -1e30f; }
   __device__ static __forceinline__ float from_float(float v) { return v; }
   // min and max of the whole group, in every lane of the row
-  // CHN: chunks of the Store in use; LANES: lanes that share the group (16, or 32 / 64 with one chunk per lane)
-  template <int CHN = 4, int LANES = 16>
   __device__ static __forceinline__ void group_minmax(const Store& st, float& lo_out, float& hi_out) {
     float lo = init_lo(), hi = init_hi();
 #pragma unroll
-    for (int k = 0; k < CHN; k++)
+    for (int k = 0; k < kQChunks; k++)
 #pragma unroll
       for (int e = 0; e < 4; e++) {
         lo = __builtin_fminf(lo, st.v[k][e]);
         hi = __builtin_fmaxf(hi, st.v[k][e]);
       }
     row_all_minmax(lo, hi);
-    rows_all_minmax<LANES>(lo, hi);
     lo_out = lo;
     hi_out = hi;
   }
@@ -353,12 +309,11 @@ template <> struct Elem<f16> {
   // min and max of the whole group, in every lane of the row: packed per-lane min / max from +-inf (the
   // start values only survive in a lane whose 16 elements are all NaN), the two halves against each other,
   // then the row reduction
-  template <int CHN = 2, int LANES = 16>
   __device__ static __forceinline__ void group_minmax(const Store& st, f16& lo_out, f16& hi_out) {
     const f16 inf = (f16)__builtin_inff();
     f16x2 l = {inf, inf}, h = {(f16)-inf, (f16)-inf};
 #pragma unroll
-    for (int k = 0; k < CHN; k++)
+    for (int k = 0; k < kQChunks; k++)
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         l = pk_min(l, st.v[k][j]);
@@ -370,7 +325,6 @@ template <> struct Elem<f16> {
     asm("v_max_f16_sdwa %0, %1, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1"
         : "=v"(hi) : "v"(h));
     row_all_minmax(lo, hi);
-    rows_all_minmax<LANES>(lo, hi);
     lo_out = lo;
     hi_out = hi;
   }
@@ -477,18 +431,16 @@ template <> struct Elem<bf16> {
     if (e & 1) st.w[k][e >> 1] |= h << 16;   // the callers set a chunk's elements in order: the even one starts the pair
     else st.w[k][e >> 1] = h;
   }
-  template <int CHN = 2, int LANES = 16>
   __device__ static __forceinline__ void group_minmax(const Store& st, float& lo_out, float& hi_out) {
     float lo = Elem<float>::init_lo(), hi = Elem<float>::init_hi();
 #pragma unroll
-    for (int k = 0; k < CHN; k++)
+    for (int k = 0; k < kQChunks; k++)
 #pragma unroll
       for (int e = 0; e < 8; e++) {
         lo = __builtin_fminf(lo, widen(st, k, e));
         hi = __builtin_fmaxf(hi, widen(st, k, e));
       }
     row_all_minmax(lo, hi);
-    rows_all_minmax<LANES>(lo, hi);
     lo_out = lo;
     hi_out = hi;
   }
@@ -939,22 +891,30 @@ __device__ __forceinline__ void dequantize_block128(const uint8_t* __restrict__ 
   }
 }
 
-// Row min/max only (the minimax entry point at D = 256).
+// Row min/max only (the minimax entry point at D = 256): a 16-lane row takes MINIMAX_ROW_GROUPS consecutive
+// groups, issues all their loads, reduces them one after the other and lets lane g store the results of group g.
+#define MINIMAX_ROW_GROUPS 4
 template <typename T>
 __device__ __forceinline__ void minimax_row(const T* __restrict__ x, int64_t N, int64_t row, int i,
                                             T* __restrict__ mn, T* __restrict__ mx) {
-#pragma unroll 2
-  for (int g = 0; g < ROW_GROUPS; g++) {
-    const int64_t n = row * ROW_GROUPS + g;
-    if (n >= N) break;
-    typename Elem<T>::Store v;
-    load_group<T>(x, N * GROUP, n, i, v);
-    T lo, hi;
-    Elem<T>::group_minmax(v, lo, hi);
-    if (i == 0) {
-      mn[n] = lo;
-      mx[n] = hi;
+  const int64_t n0 = row * MINIMAX_ROW_GROUPS;
+  typename Elem<T>::Store v[MINIMAX_ROW_GROUPS];
+#pragma unroll
+  for (int g = 0; g < MINIMAX_ROW_GROUPS; g++)
+    if (n0 + g < N) load_group<T>(x, N * GROUP, n0 + g, i, v[g]);
+  T lo_m = (T)0.0f, hi_m = (T)0.0f;
+#pragma unroll
+  for (int g = 0; g < MINIMAX_ROW_GROUPS; g++) {
+    if (n0 + g < N) {
+      T lo, hi;
+      Elem<T>::group_minmax(v[g], lo, hi);
+      lo_m = i == g ? lo : lo_m;
+      hi_m = i == g ? hi : hi_m;
     }
+  }
+  if (i < MINIMAX_ROW_GROUPS && n0 + i < N) {
+    mn[n0 + i] = lo_m;
+    mx[n0 + i] = hi_m;
   }
 }
 
@@ -973,10 +933,10 @@ __host__ __device__ constexpr int dq_supergroups(int bits) { return ROW_GROUPS /
 #define GACT_XCD_RUN_DQ 16
 #endif
 #ifndef GACT_XCD_RUN_Q_LOW
-#define GACT_XCD_RUN_Q_LOW 0 /* quantize, 1 and 2 bit */
+#define GACT_XCD_RUN_Q_LOW 0 /* quantize, 1 bit: the long one-wave workgroups gain nothing or lose (mid-sized tensors 3 %) */
 #endif
 #ifndef GACT_XCD_RUN_Q
-#define GACT_XCD_RUN_Q 128 /* quantize, 4 and 8 bit (2-4 % there; the 1 and 2 bit kernels gain nothing or lose) */
+#define GACT_XCD_RUN_Q 128 /* quantize, 2, 4 and 8 bit: 2-6 % (half 2 bit 52.7 -> 50.2 us, float 2 bit 70.1 -> 68.8 us at 134 / 103 M elements) */
 #endif
 template <uint32_t RUN>
 __device__ __forceinline__ uint32_t xcd_tile(uint32_t b, uint32_t nb) {
@@ -1002,194 +962,12 @@ __global__ void __launch_bounds__(256)
 quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
                 typename Elem<T>::Stat* __restrict__ scale_out, T* mn_io, T* mx_io, SeedArg seed_arg,
                 const float* __restrict__ noise) {
-  constexpr uint32_t RUN = BITS >= 4 ? GACT_XCD_RUN_Q : GACT_XCD_RUN_Q_LOW;
+  constexpr uint32_t RUN = BITS >= 2 ? GACT_XCD_RUN_Q : GACT_XCD_RUN_Q_LOW;
   const int64_t sg = (int64_t)xcd_tile<RUN>(blockIdx.x, gridDim.x) * (blockDim.x >> 4) + (threadIdx.x >> 4);
   if (sg * (8 / BITS) >= N) return;
   const uint64_t seed = seed_arg.value();
   quantize_supergroup<T, BITS, NOISE, GIVEN>(x, numel, N, sg, threadIdx.x & 15, packed, scale_out, mn_io, mx_io,
                                              (uint32_t)seed, (uint32_t)(seed >> 32), noise);
-}
-
-// The wide layout: one 16-byte chunk per lane and group, so GROUP / W lanes share a super-group - a whole wave
-// for float, half a wave for half and bfloat16 - and every load instruction reads whole groups.  With one
-// 16-lane row per super-group a wave of the float 1 bit kernel holds 32 KB in 128 registers per lane and the
-// kernel runs on few, long waves; here it holds 8 KB.  The row reductions are followed by one or two
-// exchanges across the rows; the byte of a column still belongs to one lane.  Same arithmetic (the same
-// Elem<T> functions on chunk 0 of a Store), same noise per element, same bytes.
-template <typename T, int BITS, int NOISE>
-__device__ __forceinline__ void quantize_supergroup_wide(const T* __restrict__ x, int64_t numel, int64_t N, int64_t sg,
-                                                         int l, uint8_t* __restrict__ packed,
-                                                         typename Elem<T>::Stat* __restrict__ scale_out,
-                                                         T* __restrict__ mn_out, T* __restrict__ mx_out, uint32_t k0,
-                                                         uint32_t k1, const float* __restrict__ noise) {
-  constexpr int WPT = 8 / BITS;
-  constexpr int QMAX = (1 << BITS) - 1;
-  constexpr int W = Elem<T>::kQWidth, LPS = GROUP / W;
-  static_assert(W == 8 || WPT >= 2, "4-column chunks pair two groups for the fast stream");
-  typedef typename Elem<T>::Stat Stat;
-  const int64_t n0 = sg * WPT;
-
-  typename Elem<T>::Store v[WPT];
-#pragma unroll
-  for (int ni = 0; ni < WPT; ni++) {
-    const int64_t n = n0 + ni;
-    if (n < N) {
-      const int64_t base = n * GROUP + W * l;
-      if (n * GROUP + GROUP <= numel) {
-        Elem<T>::load_chunk(x + base, v[ni], 0);
-      } else {
-#pragma unroll
-        for (int e = 0; e < W; e++) Elem<T>::set(v[ni], 0, e, base + e < numel ? x[base + e] : (T)0.0f);
-      }
-    }
-  }
-  Stat lo_t[WPT], hi_t[WPT], s_t[WPT];
-#pragma unroll
-  for (int ni = 0; ni < WPT; ni++) {
-    lo_t[ni] = (Stat)0.0f;
-    hi_t[ni] = (Stat)0.0f;
-    if (n0 + ni < N) Elem<T>::template group_minmax<1, LPS>(v[ni], lo_t[ni], hi_t[ni]);
-  }
-  // one scale division per lane: lane j of every row takes group j % WPT, then the row shares the results
-  {
-    const int mine = l & (WPT - 1);
-    Stat lo_m = lo_t[0], hi_m = hi_t[0];
-#pragma unroll
-    for (int ni = 1; ni < WPT; ni++) {
-      lo_m = (mine == ni) ? lo_t[ni] : lo_m;
-      hi_m = (mine == ni) ? hi_t[ni] : hi_m;
-    }
-    const Stat s_m = Elem<T>::make_scale(lo_m, hi_m, QMAX);
-    if (l < WPT && n0 + l < N) {
-      scale_out[n0 + l] = s_m;
-      mn_out[n0 + l] = Elem<T>::elem_of(lo_m);
-      if (mx_out) mx_out[n0 + l] = Elem<T>::elem_of(hi_m);
-    }
-    if (WPT == 1) {
-      s_t[0] = s_m;
-    } else {
-      s_t[0] = row_bcast<0>(s_m);
-      if (WPT > 1) s_t[1 % WPT] = row_bcast<1>(s_m);
-      if (WPT > 2) { s_t[2 % WPT] = row_bcast<2>(s_m); s_t[3 % WPT] = row_bcast<3>(s_m); }
-      if (WPT > 4) {
-        s_t[4 % WPT] = row_bcast<4>(s_m); s_t[5 % WPT] = row_bcast<5>(s_m);
-        s_t[6 % WPT] = row_bcast<6>(s_m); s_t[7 % WPT] = row_bcast<7>(s_m);
-      }
-    }
-  }
-
-  uint32_t bytes[W];
-#pragma unroll
-  for (int e = 0; e < W; e++) bytes[e] = 0;
-
-  if (NOISE == GACT_NOISE_REF) {
-#pragma unroll
-    for (int e = 0; e < W; e++) {
-      const uint64_t j = (uint64_t)sg * GROUP + W * l + e;
-      uint32_t r[4];
-#pragma unroll
-      for (int ni = 0; ni < WPT; ni++) {
-        if ((ni & 3) == 0) philox4x32<PHILOX_REF_ROUNDS>(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r);
-        if (n0 + ni < N)
-          bytes[e] |= Elem<T>::template code1<false>(v[ni], 0, e, lo_t[ni], s_t[ni], curand_uniform_map(r[ni & 3])) << (ni * BITS);
-      }
-    }
-  } else {
-    constexpr int STEP = W == 8 ? 1 : 2;   // groups whose noise is drawn together
-#pragma unroll
-    for (int g = 0; g < WPT; g += STEP) {
-      float u[STEP][W];
-      if (NOISE == GACT_NOISE_FAST) {
-        // lane l owns columns W*l ..: the lanes of the upper half of the group take the mirror image of what the
-        // lanes of the lower half draw, so both halves compute the same block
-        constexpr int HALF = LPS / 2;
-        const int lh = l & (HALF - 1);
-        const bool upper = l >= HALF;
-        if (W == 8) {
-          const uint64_t blk = (uint64_t)(n0 + g) * 16 + lh;
-          uint32_t r[4];
-          philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
-#pragma unroll
-          for (int e = 0; e < W; e++) {
-            const float d = fast_piece(r[(e >> 2) * 2], r[(e >> 2) * 2 + 1], e & 3);
-            u[0][e] = upper ? fast_mirror(d) : d;
-          }
-        } else {
-          // a Philox block feeds 8 consecutive columns = those of a pair of neighbouring lanes: the even
-          // lane computes the block of group g, the odd lane that of group g + 1, and they exchange halves
-          const bool odd = l & 1;
-          const uint64_t blk = (uint64_t)(n0 + g + (odd ? 1 : 0)) * 16 + (lh >> 1);
-          uint32_t r[4];
-          philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
-          const uint32_t ga = swap_with_neighbour(odd ? r[0] : r[2]);
-          const uint32_t gb = swap_with_neighbour(odd ? r[1] : r[3]);
-          const uint32_t a0 = odd ? ga : r[0], a1 = odd ? gb : r[1];   // group g
-          const uint32_t b0 = odd ? r[2] : ga, b1 = odd ? r[3] : gb;   // group g + 1
-#pragma unroll
-          for (int e = 0; e < W; e++) {
-            const float da = fast_piece(a0, a1, e), db = fast_piece(b0, b1, e);
-            u[0][e] = upper ? fast_mirror(da) : da;
-            u[STEP - 1][e] = upper ? fast_mirror(db) : db;
-          }
-        }
-      } else {
-#pragma unroll
-        for (int h = 0; h < STEP; h++) {
-          if (NOISE == GACT_NOISE_INJECT && n0 + g + h < N) {
-            Elem<T>::load_noise(noise + (n0 + g + h) * GROUP + W * l, u[h]);
-          } else {
-#pragma unroll
-            for (int e = 0; e < W; e++) u[h][e] = 0.5f;
-          }
-        }
-      }
-#pragma unroll
-      for (int h = 0; h < STEP; h++) {
-        const int ni = g + h;
-        if (n0 + ni < N) {
-          uint32_t c[W];
-          Elem<T>::template codes<NOISE == GACT_NOISE_CONST, false>(v[ni], 0, lo_t[ni], s_t[ni], u[h], c);
-#pragma unroll
-          for (int e = 0; e < W; e++) bytes[e] |= c[e] << (ni * BITS);
-        }
-      }
-    }
-  }
-  Elem<T>::store_codes(packed + sg * GROUP + W * l, bytes);
-}
-
-// Which (type, width) pairs take the wide layout in the single-tensor fused quantize, as bit sets of widths.
-// Measured on buffers that are cold in every cache (us, row layout -> wide layout): float 1 bit 36.5 -> 35.0 at
-// 43 M elements, even at 17 - 75 M, either sign from 103 M on (the launch keeps the row layout there);
-// bfloat16 1 bit 30.0 -> 27.3 at 43 M, 75.9 -> 70.8 at 134 M.  Every other pair loses 2-30 % (half 1 bit
-// 65.5 -> 69.5, float 4 bit 92.9 -> 106.4 at 134 M): their rows already hold 8 KB per wave or less.
-#ifndef GACT_Q_WIDE_MASK_F32
-#define GACT_Q_WIDE_MASK_F32 0x1
-#endif
-#ifndef GACT_Q_WIDE_MASK_F16
-#define GACT_Q_WIDE_MASK_F16 0x0
-#endif
-#ifndef GACT_Q_WIDE_MASK_BF16
-#define GACT_Q_WIDE_MASK_BF16 0x1
-#endif
-template <typename T>
-__host__ __device__ constexpr bool quantize_is_wide(int bits) {
-  return ((Elem<T>::kDtype == GACT_F32 ? GACT_Q_WIDE_MASK_F32
-                                        : Elem<T>::kDtype == GACT_F16 ? GACT_Q_WIDE_MASK_F16 : GACT_Q_WIDE_MASK_BF16) &
-          bits) != 0;
-}
-
-template <typename T, int BITS, int NOISE>
-__global__ void __launch_bounds__(256)
-quantize_wide_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
-                     typename Elem<T>::Stat* __restrict__ scale_out, T* __restrict__ mn_out, T* __restrict__ mx_out,
-                     SeedArg seed_arg, const float* __restrict__ noise) {
-  constexpr int LPS = GROUP / Elem<T>::kQWidth;
-  const int64_t sg = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / LPS;
-  if (sg * (8 / BITS) >= N) return;
-  const uint64_t seed = seed_arg.value();
-  quantize_supergroup_wide<T, BITS, NOISE>(x, numel, N, sg, threadIdx.x % LPS, packed, scale_out, mn_out, mx_out,
-                                           (uint32_t)seed, (uint32_t)(seed >> 32), noise);
 }
 
 template <typename T, int BITS>
@@ -1207,8 +985,8 @@ dequantize_kernel(const uint8_t* __restrict__ packed, const typename Elem<T>::St
 template <typename T>
 __global__ void __launch_bounds__(256)
 minimax256_kernel(const T* __restrict__ x, int64_t N, T* __restrict__ mn, T* __restrict__ mx) {
-  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
-  if (row * ROW_GROUPS >= N) return;
+  const int64_t row = (int64_t)xcd_tile<GACT_XCD_RUN_Q>(blockIdx.x, gridDim.x) * (blockDim.x >> 4) + (threadIdx.x >> 4);
+  if (row * MINIMAX_ROW_GROUPS >= N) return;
   minimax_row<T>(x, N, row, threadIdx.x & 15, mn, mx);
 }
 
@@ -1943,15 +1721,15 @@ inline void row_grid(int64_t rows, dim3* grid, dim3* block, int threads = 256) {
 // Workgroup size of the quantize kernel.  A row's work grows with 8/bits groups; the long-running
 // low-width rows schedule better as single-wave workgroups (measured: float 2 bit 5.7 -> 6.2 TB/s,
 // 1 bit 5.4 -> 6.0 TB/s), the short high-width ones as four waves.
-#ifndef GACT_Q_WIDE_F32
-#define GACT_Q_WIDE_F32 8
+#ifndef GACT_Q_BLOCK256_F32
+#define GACT_Q_BLOCK256_F32 8 /* width from which float rows run in four-wave workgroups */
 #endif
-#ifndef GACT_Q_WIDE_F16
-#define GACT_Q_WIDE_F16 4
+#ifndef GACT_Q_BLOCK256_F16
+#define GACT_Q_BLOCK256_F16 4
 #endif
 inline int quantize_threads(int bits, size_t elem_size) {
-  const int wide_from = elem_size == 4 ? GACT_Q_WIDE_F32 : GACT_Q_WIDE_F16;
-  return bits >= wide_from ? 256 : 64;
+  const int from = elem_size == 4 ? GACT_Q_BLOCK256_F32 : GACT_Q_BLOCK256_F16;
+  return bits >= from ? 256 : 64;
 }
 inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8 / bits); }
 
@@ -1985,30 +1763,6 @@ template <typename T, int BITS, bool GIVEN>
 int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, typename Elem<T>::Stat* scale, T* mn, T* mx,
                     int noise_mode,
                     SeedArg seed, const float* noise, hipStream_t stream) {
-  // float: only below 50 M elements (43 M: 36.5 -> 35.0 us, 75 M: even, 103 M: 72.2 -> 73.8 us) - the shorter
-  // waves shorten the tail of a mid-sized launch, the long ones stream a little better once the tail is small
-  const bool wide_here = Elem<T>::kDtype != GACT_F32 || N < kCapFromGroups;
-  if constexpr (!GIVEN && quantize_is_wide<T>(BITS) && (Elem<T>::kQWidth == 8 || BITS < 8)) if (wide_here) {
-    const int64_t per_block = 256 / (GROUP / Elem<T>::kQWidth);
-    const dim3 wgrid((unsigned)((supergroups(N, BITS) + per_block - 1) / per_block)), wblock(256);
-    switch (noise_mode) {
-      case GACT_NOISE_CONST:
-        hipLaunchKernelGGL((quantize_wide_kernel<T, BITS, GACT_NOISE_CONST>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
-        break;
-      case GACT_NOISE_INJECT:
-        hipLaunchKernelGGL((quantize_wide_kernel<T, BITS, GACT_NOISE_INJECT>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
-        break;
-      case GACT_NOISE_REF:
-        hipLaunchKernelGGL((quantize_wide_kernel<T, BITS, GACT_NOISE_REF>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
-        break;
-      case GACT_NOISE_FAST:
-        hipLaunchKernelGGL((quantize_wide_kernel<T, BITS, GACT_NOISE_FAST>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
-        break;
-      default:
-        return GACT_EINVAL;
-    }
-    return launch_status();
-  }
   dim3 grid, block;
   row_grid(supergroups(N, BITS), &grid, &block, quantize_threads(BITS, sizeof(T)));
   // the reference stream's one Philox block per byte makes the kernel instruction-bound: it wants every wave
@@ -2175,7 +1929,7 @@ int gact_minimax(const void* data, int dtype, int64_t N, int64_t D, void* mn, vo
   hipStream_t s = (hipStream_t)stream;
   if (D == GROUP && aligned16(data)) {
     dim3 grid, block;
-    row_grid((N + ROW_GROUPS - 1) / ROW_GROUPS, &grid, &block);
+    row_grid((N + MINIMAX_ROW_GROUPS - 1) / MINIMAX_ROW_GROUPS, &grid, &block);
     if (dtype == GACT_F32)
       hipLaunchKernelGGL((minimax256_kernel<float>), grid, block, 0, s, (const float*)data, N, (float*)mn, (float*)mx);
     else
