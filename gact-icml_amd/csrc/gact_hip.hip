@@ -144,20 +144,28 @@ __device__ __forceinline__ uint32_t rint_clamp0(float z) {
   return c;
 }
 
-// The same code taken from y directly, in two instructions instead of three, for 0 <= y < 2^22, negative y,
-// +-inf and NaN: y + (2^23 - 0.5) is rounded to a float whose unit in the last place is 1, i.e. to
-// 2^23 + rint(y - 0.5) (y - 0.5 itself is exact for 0.5 <= y < 2^23, so rounding the sum once equals
-// rounding the difference and then the integer; ties go to even in both since 2^23 is even), and the
-// integer sits in the low mantissa bits.  The median clamps to [2^23, 2^23 + 0x3fffff]: everything below
-// 0.5, negative or NaN gives 0 like the reference's fmax, and +inf (a half scale that overflowed) gives
-// low bits of all ones like the reference's saturated 0x7fffffff.  The bits above the code (0x4B...) never
-// reach the low 8 bits a byte keeps of a code shifted left by at most 7.
+// The same code read off the float.  For 0.5 <= y < 2^22, y - 0.5 is exact and adding 1.5 * 2^23 rounds it to
+// 1.5 * 2^23 + rint(y - 0.5): in that binade a float's unit in the last place is 1, the constant is even, so
+// ties go to even exactly as rint's do, and the integer sits in the low mantissa bits.  For 0 <= y < 0.5 the
+// difference lies in [-0.5, 0) (possibly rounded, which cannot take it out of that interval) and the sum rounds
+// to the constant itself: code 0, the reference's fmax.  NaN stays NaN, whose low byte is 0: code 0 as well.
+// Two additions; the bits above the code (0x4B4...) never reach the low 8 bits a byte keeps of a code shifted
+// left by at most 7.  NOT valid for negative y (the callers' y is a sum of non-negative terms: with the group's own
+// minimum no element lies below it) and for +inf, whose bits have a zero low byte where the reference's saturated
+// conversion has 0xff: the one caller that can meet +inf (a half scale that overflowed) repairs those groups
+// afterwards (quantize_supergroup).
+__device__ __forceinline__ uint32_t code_bits_of(float y) {
+  const float z = y - 0.5f;
+  return __builtin_bit_cast(uint32_t, z + 12582912.0f);
+}
+// The same for any y: y + (2^23 - 0.5) rounds to 2^23 + rint(y - 0.5) in one step, and the median clamps to
+// [2^23, 2^23 + 0x3fffff]: everything below 0.5, negative or NaN gives 0, +inf gives low bits of all ones.
 __device__ __forceinline__ uint32_t clamp_code_bits(float w) {
   float c;
   asm("v_med3_f32 %0, %1, %2, %3" : "=v"(c) : "v"(w), "v"(8388608.0f), "v"(12582911.0f));
   return __builtin_bit_cast(uint32_t, c);
 }
-__device__ __forceinline__ uint32_t code_bits_of(float y) { return clamp_code_bits(y + 8388607.5f); }
+__device__ __forceinline__ uint32_t code_bits_of_any(float y) { return clamp_code_bits(y + 8388607.5f); }
 
 // Correctly rounded c / s from the correctly rounded reciprocal r = RN(1/s) (Markstein): q = RN(c*r),
 // e = c - s*q exactly (one FMA), result RN(q + e*r).  Valid for finite nonzero s with a normal quotient;
@@ -237,6 +245,11 @@ template <> struct Elem<float> {
 #pragma unroll
     for (int e = 0; e < 4; e++) c[e] = code1<ANY>(st, k, e, mn, s, u[e]);
   }
+  // a float scale is never infinite (the denominator is at least 2e-6) and with the group's own min and max the
+  // sum stays finite: nothing to repair
+  static constexpr bool kRepairsInfiniteScale = false;
+  __device__ static __forceinline__ bool scale_is_inf(float) { return false; }
+  __device__ static __forceinline__ bool above(const Store&, int, int, float) { return false; }
 
   // ---- dequantize: out = float(code) / scale + min ----
   struct Dq { float s, r, mn; bool fast; };
@@ -346,13 +359,15 @@ template <> struct Elem<f16> {
   }
   // half subtraction and half product (each rounded to half), then float: y = float(p) + u,
   // code = rint(max(y - 0.5, 0)).  |y| <= 65505 or y is infinite or NaN whatever min and scale are, so the
-  // code is always read off the float (code_bits_of); ANY changes nothing here.
+  // code is always read off the float.  ANY = true (min and scale from the caller): y may be negative or +inf,
+  // the clamping form takes both.  ANY = false: y >= 0, and where it is +inf (the scale overflowed to inf)
+  // the caller repairs the group afterwards.
   template <bool ANY>
   __device__ static __forceinline__ uint32_t code1(const Store& st, int k, int e, f16 mn, f16 s, float u) {
     f16 t = st.v[k][e >> 1][e & 1] - mn;
     f16 p = t * s;
     float y = (float)p + u;
-    return code_bits_of(y);
+    return ANY ? code_bits_of_any(y) : code_bits_of(y);
   }
   template <bool CONST_NOISE, bool ANY>
   __device__ static __forceinline__ void codes(const Store& st, int k, f16 mn, f16 s, const float (&u)[8],
@@ -365,15 +380,29 @@ template <> struct Elem<f16> {
       if (CONST_NOISE) {
         // u = 0.5: float(p) + 0.5 and the following - 0.5 are both exact for every half p (at most 24
         // significant bits between 2^-1 and p's last bit), so y - 0.5 == float(p) and the code is
-        // rint(float(p)): float(p) + 2^23 rounds to 2^23 + rint(float(p))
-        c[2 * j] = clamp_code_bits(widen_add_lo(p, 8388608.0f));
-        c[2 * j + 1] = clamp_code_bits(widen_add_hi(p, 8388608.0f));
+        // rint(float(p)): float(p) plus the constant rounds to the constant + rint(float(p))
+        if (ANY) {
+          c[2 * j] = clamp_code_bits(widen_add_lo(p, 8388608.0f));
+          c[2 * j + 1] = clamp_code_bits(widen_add_hi(p, 8388608.0f));
+        } else {
+          c[2 * j] = __builtin_bit_cast(uint32_t, widen_add_lo(p, 12582912.0f));
+          c[2 * j + 1] = __builtin_bit_cast(uint32_t, widen_add_hi(p, 12582912.0f));
+        }
+      } else if (ANY) {
+        c[2 * j] = code_bits_of_any(widen_add_lo(p, u[2 * j]));
+        c[2 * j + 1] = code_bits_of_any(widen_add_hi(p, u[2 * j + 1]));
       } else {
         c[2 * j] = code_bits_of(widen_add_lo(p, u[2 * j]));
         c[2 * j + 1] = code_bits_of(widen_add_hi(p, u[2 * j + 1]));
       }
     }
   }
+  // Where the scale is +inf every element above the minimum has an infinite product, whose code the reference
+  // saturates to 0x7fffffff: all ones from the element's field upwards.  (An element equal to the minimum gives
+  // 0 * inf = NaN: code 0.)  code_bits_of leaves 0 in both cases; this adds the ones.
+  static constexpr bool kRepairsInfiniteScale = true;
+  __device__ static __forceinline__ bool scale_is_inf(f16 s) { return __builtin_isinf((float)s); }
+  __device__ static __forceinline__ bool above(const Store& st, int k, int e, f16 mn) { return st.v[k][e >> 1][e & 1] > mn; }
 
   // ---- dequantize: half(code) / scale is a float division rounded to half; the sum is rounded to half ----
   struct Dq { float s, r; f16 mn; bool fast; };
@@ -459,6 +488,9 @@ template <> struct Elem<bf16> {
 #pragma unroll
     for (int e = 0; e < 8; e++) c[e] = code1<ANY>(st, k, e, mn, s, u[e]);
   }
+  static constexpr bool kRepairsInfiniteScale = false;
+  __device__ static __forceinline__ bool scale_is_inf(float) { return false; }
+  __device__ static __forceinline__ bool above(const Store&, int, int, float) { return false; }
   __device__ static __forceinline__ bf16 finish(float q, float mn) { return (bf16)(q + mn); }
   __device__ static __forceinline__ uint32_t table_entry(float c, float s, float mn) {
     return (uint32_t)__builtin_bit_cast(uint16_t, (bf16)(c / s + mn));
@@ -569,128 +601,158 @@ __device__ __forceinline__ void fast_noise(int64_t n, int i, uint32_t k0, uint32
 }
 
 // ------------------------------------------------------------------------------------------------
-// Quantize one super-group (one 16-lane row).
+// Quantize SGR consecutive super-groups (one 16-lane row): all their groups are loaded first, reduced, and share
+// one scale division per lane; the codes then go out super-group by super-group.
 //   GIVEN = false: min/max are reduced here (fused minimax + scale + pack, one read of x).
 //   GIVEN = true : min/max are read from mn_io / mx_io (the pack entry point's contract).
 // Codes follow quantization_cuda_kernel.cu:38-71; see Elem<T>::code1 for the arithmetic.
 // ------------------------------------------------------------------------------------------------
-template <typename T, int BITS, int NOISE, bool GIVEN>
-__device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int64_t numel, int64_t N, int64_t sg,
+template <typename T, int BITS, int NOISE, bool GIVEN, int SGR = 1>
+__device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int64_t numel, int64_t N, int64_t sg0,
                                                     int i, uint8_t* __restrict__ packed,
                                                     typename Elem<T>::Stat* __restrict__ scale_out,
                                                     T* mn_io, T* mx_io, uint32_t k0, uint32_t k1,
                                                     const float* __restrict__ noise) {
   constexpr int WPT = 8 / BITS;
+  constexpr int GPR = SGR * WPT;   // groups of the row
+  static_assert(GPR == 1 || GPR == 2 || GPR == 4 || GPR == 8, "a row holds 1, 2, 4 or 8 groups");
   constexpr int QMAX = (1 << BITS) - 1;
   constexpr int CH = Elem<T>::kQChunks, W = Elem<T>::kQWidth;
-  const int64_t n0 = sg * WPT;
+  const int64_t n0 = sg0 * WPT;
 
-  typename Elem<T>::Store v[WPT];
+  typename Elem<T>::Store v[GPR];
   typedef typename Elem<T>::Stat Stat;
-  Stat lo_t[WPT], hi_t[WPT], s_t[WPT];
+  Stat lo_t[GPR], hi_t[GPR], s_t[GPR];
 #pragma unroll
-  for (int ni = 0; ni < WPT; ni++) {
-    if (n0 + ni < N) load_group<T>(x, numel, n0 + ni, i, v[ni]);
+  for (int g = 0; g < GPR; g++) {
+    if (n0 + g < N) load_group<T>(x, numel, n0 + g, i, v[g]);
   }
 #pragma unroll
-  for (int ni = 0; ni < WPT; ni++) {
-    const int64_t n = n0 + ni;
-    lo_t[ni] = (Stat)0.0f;
-    hi_t[ni] = (Stat)0.0f;
+  for (int g = 0; g < GPR; g++) {
+    const int64_t n = n0 + g;
+    lo_t[g] = (Stat)0.0f;
+    hi_t[g] = (Stat)0.0f;
     if (n < N) {
       if (GIVEN) {
-        lo_t[ni] = Elem<T>::stat_of(mn_io[n]);
-        hi_t[ni] = Elem<T>::stat_of(mx_io[n]);
+        lo_t[g] = Elem<T>::stat_of(mn_io[n]);
+        hi_t[g] = Elem<T>::stat_of(mx_io[n]);
       } else {
-        Elem<T>::group_minmax(v[ni], lo_t[ni], hi_t[ni]);
+        Elem<T>::group_minmax(v[g], lo_t[g], hi_t[g]);
       }
     }
   }
-  // one scale division per lane: lane j of the row takes group j % WPT, then the row shares the results
+  // one scale division per lane: lane j of the row takes group j % GPR, then the row shares the results
   {
-    const int mine = i & (WPT - 1);
+    const int mine = i & (GPR - 1);
     Stat lo_m = lo_t[0], hi_m = hi_t[0];
 #pragma unroll
-    for (int ni = 1; ni < WPT; ni++) {
-      lo_m = (mine == ni) ? lo_t[ni] : lo_m;
-      hi_m = (mine == ni) ? hi_t[ni] : hi_m;
+    for (int g = 1; g < GPR; g++) {
+      lo_m = (mine == g) ? lo_t[g] : lo_m;
+      hi_m = (mine == g) ? hi_t[g] : hi_m;
     }
     const Stat s_m = Elem<T>::make_scale(lo_m, hi_m, QMAX);
-    if (i < WPT && n0 + i < N) {
+    if (i < GPR && n0 + i < N) {
       scale_out[n0 + i] = s_m;
       if (!GIVEN) {
         mn_io[n0 + i] = Elem<T>::elem_of(lo_m);
         if (mx_io) mx_io[n0 + i] = Elem<T>::elem_of(hi_m);
       }
     }
-    if (WPT == 1) {
+    if (GPR == 1) {
       s_t[0] = s_m;
     } else {
       s_t[0] = row_bcast<0>(s_m);
-      if (WPT > 1) s_t[1 % WPT] = row_bcast<1>(s_m);
-      if (WPT > 2) { s_t[2 % WPT] = row_bcast<2>(s_m); s_t[3 % WPT] = row_bcast<3>(s_m); }
-      if (WPT > 4) {
-        s_t[4 % WPT] = row_bcast<4>(s_m); s_t[5 % WPT] = row_bcast<5>(s_m);
-        s_t[6 % WPT] = row_bcast<6>(s_m); s_t[7 % WPT] = row_bcast<7>(s_m);
+      if (GPR > 1) s_t[1 % GPR] = row_bcast<1>(s_m);
+      if (GPR > 2) { s_t[2 % GPR] = row_bcast<2>(s_m); s_t[3 % GPR] = row_bcast<3>(s_m); }
+      if (GPR > 4) {
+        s_t[4 % GPR] = row_bcast<4>(s_m); s_t[5 % GPR] = row_bcast<5>(s_m);
+        s_t[6 % GPR] = row_bcast<6>(s_m); s_t[7 % GPR] = row_bcast<7>(s_m);
       }
     }
   }
 
-  uint32_t bytes[CH][W];
 #pragma unroll
-  for (int k = 0; k < CH; k++)
-#pragma unroll
-    for (int e = 0; e < W; e++) bytes[k][e] = 0;
-
-  if (NOISE == GACT_NOISE_REF) {
-    // one Philox state per output byte j: key = seed, counter = (draw/4, 0, j lo, j hi)
+  for (int q = 0; q < SGR; q++) {
+    const int64_t sg = sg0 + q;
+    if (q == 0 || sg * WPT < N) {
+    uint32_t bytes[CH][W];
 #pragma unroll
     for (int k = 0; k < CH; k++)
 #pragma unroll
-      for (int e = 0; e < W; e++) {
-        const uint64_t j = (uint64_t)sg * GROUP + chunk_col<T>(k, i) + e;
-        uint32_t r[4];
+      for (int e = 0; e < W; e++) bytes[k][e] = 0;
+
+    if (NOISE == GACT_NOISE_REF) {
+      // one Philox state per output byte j: key = seed, counter = (draw/4, 0, j lo, j hi)
 #pragma unroll
-        for (int ni = 0; ni < WPT; ni++) {
-          if ((ni & 3) == 0) philox4x32<PHILOX_REF_ROUNDS>(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r);
-          if (n0 + ni < N) {
-            float u = curand_uniform_map(r[ni & 3]);
-            bytes[k][e] |= Elem<T>::template code1<GIVEN>(v[ni], k, e, lo_t[ni], s_t[ni], u) << (ni * BITS);
-          }
-        }
-      }
-  } else {
+      for (int k = 0; k < CH; k++)
 #pragma unroll
-    for (int ni = 0; ni < WPT; ni++) {
-      const int64_t n = n0 + ni;
-      if (n < N) {
-        float u[CH][W];
-        if (NOISE == GACT_NOISE_FAST) {
-          fast_noise<T>(n, i, k0, k1, u);
-        } else {
+        for (int e = 0; e < W; e++) {
+          const uint64_t j = (uint64_t)sg * GROUP + chunk_col<T>(k, i) + e;
+          uint32_t r[4];
 #pragma unroll
-          for (int k = 0; k < CH; k++) {
-            if (NOISE == GACT_NOISE_INJECT) {
-              Elem<T>::load_noise(noise + n * GROUP + chunk_col<T>(k, i), u[k]);
-            } else {
-#pragma unroll
-              for (int e = 0; e < W; e++) u[k][e] = 0.5f;
+          for (int ni = 0; ni < WPT; ni++) {
+            const int g = q * WPT + ni;
+            if ((ni & 3) == 0) philox4x32<PHILOX_REF_ROUNDS>(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r);
+            if (n0 + g < N) {
+              float u = curand_uniform_map(r[ni & 3]);
+              bytes[k][e] |= Elem<T>::template code1<GIVEN>(v[g], k, e, lo_t[g], s_t[g], u) << (ni * BITS);
             }
           }
         }
+    } else {
 #pragma unroll
-        for (int k = 0; k < CH; k++) {
-          uint32_t c[W];
-          Elem<T>::template codes<NOISE == GACT_NOISE_CONST, GIVEN>(v[ni], k, lo_t[ni], s_t[ni], u[k], c);
+      for (int ni = 0; ni < WPT; ni++) {
+        const int g = q * WPT + ni;
+        const int64_t n = n0 + g;
+        if (n < N) {
+          float u[CH][W];
+          if (NOISE == GACT_NOISE_FAST) {
+            fast_noise<T>(n, i, k0, k1, u);
+          } else {
 #pragma unroll
-          for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (ni * BITS);
+            for (int k = 0; k < CH; k++) {
+              if (NOISE == GACT_NOISE_INJECT) {
+                Elem<T>::load_noise(noise + n * GROUP + chunk_col<T>(k, i), u[k]);
+              } else {
+#pragma unroll
+                for (int e = 0; e < W; e++) u[k][e] = 0.5f;
+              }
+            }
+          }
+#pragma unroll
+          for (int k = 0; k < CH; k++) {
+            uint32_t c[W];
+            Elem<T>::template codes<NOISE == GACT_NOISE_CONST, GIVEN>(v[g], k, lo_t[g], s_t[g], u[k], c);
+#pragma unroll
+            for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (ni * BITS);
+          }
         }
       }
     }
-  }
 
+    if (Elem<T>::kRepairsInfiniteScale && !GIVEN) {
+      // rare: a scale of the super-group overflowed to +inf (see Elem<T>::kRepairsInfiniteScale)
+      bool any_inf = false;
 #pragma unroll
-  for (int k = 0; k < CH; k++) Elem<T>::store_codes(packed + sg * GROUP + chunk_col<T>(k, i), bytes[k]);
+      for (int ni = 0; ni < WPT; ni++) any_inf |= Elem<T>::scale_is_inf(s_t[q * WPT + ni]);
+      if (__builtin_amdgcn_ballot_w64(any_inf) != 0) {
+#pragma unroll
+        for (int ni = 0; ni < WPT; ni++) {
+          const int g = q * WPT + ni;
+          if (n0 + g < N && Elem<T>::scale_is_inf(s_t[g])) {
+#pragma unroll
+            for (int k = 0; k < CH; k++)
+#pragma unroll
+              for (int e = 0; e < W; e++)
+                if (Elem<T>::above(v[g], k, e, lo_t[g])) bytes[k][e] |= 0xffffffffu << (ni * BITS);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < CH; k++) Elem<T>::store_codes(packed + sg * GROUP + chunk_col<T>(k, i), bytes[k]);
+    }
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -856,8 +918,9 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
 }
 
 // Batched launch: a block owns 128 consecutive groups of one tensor whatever the width, so the grid does
-// not depend on the widths.  Quantize: the 16*BITS super-groups of the block go round-robin over the 16
-// rows, so that every pass of the block reads one contiguous stretch.
+// not depend on the widths.  Quantize: each of the workgroup's 16 rows takes 8 consecutive groups - BITS
+// super-groups - in one go: no loop, 16 KB (half) in flight per wave at every width, one scale division per
+// lane and 8 groups.
 template <typename T, int BITS, int NOISE>
 __device__ __forceinline__ void quantize_block128(const T* __restrict__ x, int64_t numel, int64_t N, int64_t lb,
                                                   uint8_t* __restrict__ packed,
@@ -865,12 +928,17 @@ __device__ __forceinline__ void quantize_block128(const T* __restrict__ x, int64
                                                   T* __restrict__ mn_out, uint64_t seed) {
   constexpr int WPT = 8 / BITS;
   const int row = threadIdx.x >> 4, i = threadIdx.x & 15;
+  const int64_t sg0 = (lb * 16 + row) * BITS;
+  if (NOISE == GACT_NOISE_REF) {
+    // one Philox block per output byte: far too much code to lay out for 8 groups at once; super-group by super-group
 #pragma unroll 1
-  for (int it = 0; it < BITS; it++) {
-    const int64_t sg = lb * (16 * BITS) + it * 16 + row;
-    if (sg * WPT < N)
-      quantize_supergroup<T, BITS, NOISE, false>(x, numel, N, sg, i, packed, scale_out, mn_out, (T*)nullptr,
-                                                 (uint32_t)seed, (uint32_t)(seed >> 32), nullptr);
+    for (int q = 0; q < BITS; q++)
+      if ((sg0 + q) * WPT < N)
+        quantize_supergroup<T, BITS, NOISE, false, 1>(x, numel, N, sg0 + q, i, packed, scale_out, mn_out, (T*)nullptr,
+                                                      (uint32_t)seed, (uint32_t)(seed >> 32), nullptr);
+  } else if (sg0 * WPT < N) {
+    quantize_supergroup<T, BITS, NOISE, false, BITS>(x, numel, N, sg0, i, packed, scale_out, mn_out, (T*)nullptr,
+                                                     (uint32_t)seed, (uint32_t)(seed >> 32), nullptr);
   }
 }
 // Dequantize: two workgroups share a block of 128 groups, 8 units of 8 groups each, so that a unit slot
@@ -932,6 +1000,12 @@ __host__ __device__ constexpr int dq_supergroups(int bits) { return ROW_GROUPS /
 #ifndef GACT_XCD_RUN_DQ
 #define GACT_XCD_RUN_DQ 16
 #endif
+#ifndef GACT_XCD_RUN_DQB
+#define GACT_XCD_RUN_DQB 16 /* batched dequantize */
+#endif
+#ifndef GACT_XCD_RUN_QB
+#define GACT_XCD_RUN_QB 16 /* batched quantize: 4-6 % over the plain order at every width (120 half tensors, 1.83 G elements) */
+#endif
 #ifndef GACT_XCD_RUN_Q_LOW
 #define GACT_XCD_RUN_Q_LOW 0 /* quantize, 1 bit: the long one-wave workgroups gain nothing or lose (mid-sized tensors 3 %) */
 #endif
@@ -956,18 +1030,38 @@ struct SeedArg {
   __device__ __forceinline__ uint64_t value() const { return add ? seed + *add : seed; }
 };
 
-// One super-group per 16-lane row: short waves, many of them.
+// Geometry of the single-tensor quantize launch for an element type and width: super-groups per row (a row always
+// loads all its groups before it reduces them), threads per workgroup, and the XCD-aware run of tiles.
+// Overridable at compile time for experiments: -DGACT_QGEOM_<F32|F16|BF16>_<bits>=sgr*10000+threads*... see q_geom.
+struct QGeom { int sgr, threads, run; };
+#ifndef GACT_QGEOM_F16
+#define GACT_QGEOM_F16 {{1, 64, 0}, {1, 64, 128}, {1, 256, 128}, {1, 256, 128}}
+#endif
+#ifndef GACT_QGEOM_BF16
+#define GACT_QGEOM_BF16 {{1, 64, 0}, {1, 64, 128}, {1, 256, 128}, {1, 256, 128}}
+#endif
+#ifndef GACT_QGEOM_F32
+#define GACT_QGEOM_F32 {{1, 64, 0}, {1, 64, 128}, {1, 64, 128}, {1, 256, 128}}
+#endif
+template <typename T>
+__host__ __device__ constexpr QGeom q_geom(int bits) {
+  constexpr QGeom f32[4] = GACT_QGEOM_F32, f16[4] = GACT_QGEOM_F16, b16[4] = GACT_QGEOM_BF16;
+  const int k = bits == 1 ? 0 : bits == 2 ? 1 : bits == 4 ? 2 : 3;
+  return Elem<T>::kDtype == GACT_F32 ? f32[k] : Elem<T>::kDtype == GACT_F16 ? f16[k] : b16[k];
+}
+
 template <typename T, int BITS, int NOISE, bool GIVEN>
 __global__ void __launch_bounds__(256)
 quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
                 typename Elem<T>::Stat* __restrict__ scale_out, T* mn_io, T* mx_io, SeedArg seed_arg,
                 const float* __restrict__ noise) {
-  constexpr uint32_t RUN = BITS >= 2 ? GACT_XCD_RUN_Q : GACT_XCD_RUN_Q_LOW;
-  const int64_t sg = (int64_t)xcd_tile<RUN>(blockIdx.x, gridDim.x) * (blockDim.x >> 4) + (threadIdx.x >> 4);
-  if (sg * (8 / BITS) >= N) return;
+  constexpr QGeom G = q_geom<T>(BITS);
+  constexpr int SGR = NOISE == GACT_NOISE_REF ? 1 : G.sgr;   // the reference stream's code is too long to lay out several times
+  const int64_t sg0 = ((int64_t)xcd_tile<(uint32_t)G.run>(blockIdx.x, gridDim.x) * (blockDim.x >> 4) + (threadIdx.x >> 4)) * SGR;
+  if (sg0 * (8 / BITS) >= N) return;
   const uint64_t seed = seed_arg.value();
-  quantize_supergroup<T, BITS, NOISE, GIVEN>(x, numel, N, sg, threadIdx.x & 15, packed, scale_out, mn_io, mx_io,
-                                             (uint32_t)seed, (uint32_t)(seed >> 32), noise);
+  quantize_supergroup<T, BITS, NOISE, GIVEN, SGR>(x, numel, N, sg0, threadIdx.x & 15, packed, scale_out, mn_io, mx_io,
+                                                  (uint32_t)seed, (uint32_t)(seed >> 32), noise);
 }
 
 template <typename T, int BITS>
@@ -1507,44 +1601,32 @@ calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, cons
 // ------------------------------------------------------------------------------------------------
 // The workspace of a batched launch (device memory the caller brings, or the library's static array):
 //   BatchHeader                      what the plan found
-//   int32 tensor_class_off[L]        blocks of earlier tensors of the same class
-//   int32 block_tensor[total_blocks] tensor of every block of the grid (dequantize: one launch over all blocks)
-//   int32x2 class_list[total_blocks] the blocks sorted by class, as (tensor, block within the tensor): the quantize
-//                                    kernel of a class walks its own stretch of this list and nothing else
-// A class is an (element type, width) pair: 3 types x 4 widths.
-#define BATCH_CLASSES 12
+//   int32 block_tensor[total_blocks] tensor of every block of the grid
 struct BatchHeader {
-  int64_t need;                        // arena bytes the table needs
-  int64_t ok;                          // 1: every width valid and need <= capacity
-  int64_t tensors_at[4];               // tensors at width 1, 2, 4, 8
-  int64_t reserved[2];
-  int64_t class_count[BATCH_CLASSES];  // blocks per class
-  int64_t class_start[BATCH_CLASSES];  // first entry of the class in class_list
+  int64_t need;            // arena bytes the table needs
+  int64_t ok;              // 1: every width and element type valid and need <= capacity
+  int64_t tensors_at[4];   // tensors at width 1, 2, 4, 8
+  int64_t reserved[26];
 };
 static_assert(sizeof(BatchHeader) == 256, "the header is 32 int64");
 struct BatchWorkspace {
   BatchHeader* hdr;
-  int32_t* tensor_class_off;
   int32_t* block_tensor;
-  int2* class_list;
 };
 __host__ __device__ inline int64_t batch_workspace_need(int64_t L, int64_t total_blocks) {
-  return (int64_t)sizeof(BatchHeader) + ((L + 63) / 64 * 64) * 4 + ((total_blocks + 1) / 2 * 2) * 4 + total_blocks * 8;
+  (void)L;
+  return (int64_t)sizeof(BatchHeader) + (total_blocks + 3) / 4 * 16;
 }
-__host__ __device__ inline BatchWorkspace batch_workspace(void* base, int64_t L, int64_t total_blocks) {
+__host__ __device__ inline BatchWorkspace batch_workspace(void* base) {
   BatchWorkspace w;
-  uint8_t* p = (uint8_t*)base;
-  w.hdr = (BatchHeader*)p;
-  w.tensor_class_off = (int32_t*)(p + sizeof(BatchHeader));
-  w.block_tensor = w.tensor_class_off + (L + 63) / 64 * 64;
-  w.class_list = (int2*)(w.block_tensor + (total_blocks + 1) / 2 * 2);  // stays 8-byte aligned
+  w.hdr = (BatchHeader*)base;
+  w.block_tensor = (int32_t*)((uint8_t*)base + sizeof(BatchHeader));
   return w;
 }
 __device__ __forceinline__ int width_index(int bits) { return bits == 1 ? 0 : bits == 2 ? 1 : bits == 4 ? 2 : 3; }
 
-// One wave: lane l sizes tensors l, l+64, ...; running offsets are carried across rounds of 64 with wave-wide
-// inclusive scans - one for the packed-arena offsets, one per class for the position of a tensor's blocks
-// among the blocks of its class.
+// One wave: lane l sizes tensors l, l+64, ...; the running packed-arena offset is carried across rounds of 64
+// with a wave-wide inclusive scan.
 __global__ void __launch_bounds__(64)
 batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int L, int64_t capacity,
                   BatchWorkspace ws) {
@@ -1552,25 +1634,19 @@ batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int
   int64_t base = 0;
   int bad = 0;
   int cnt[4] = {0, 0, 0, 0};
-  int class_base[BATCH_CLASSES];
-#pragma unroll
-  for (int c = 0; c < BATCH_CLASSES; c++) class_base[c] = 0;
   for (int t0 = 0; t0 < L; t0 += 64) {
     const int t = t0 + lane;
     int64_t bytes = 0;
-    int cls = -1, nb = 0;
     if (t < L) {
       int bt = bits[t];
       if (!(bt == 1 || bt == 2 || bt == 4 || bt == 8)) { bad = 1; bt = 8; }
-      int dt = table[t].dtype;
-      if (dt < 0 || dt > 2) { bad = 1; dt = 0; }
+      const int dt = table[t].dtype;
+      if (dt < 0 || dt > 2) bad = 1;
       cnt[width_index(bt)]++;
-      cls = dt * 4 + width_index(bt);
       const int wpt = 8 / bt;
       const int64_t N = (table[t].numel + GROUP - 1) / GROUP;
       const int64_t n_round = (N + wpt - 1) / wpt * wpt;
       bytes = ((int64_t)bt * n_round * (GROUP / 8) + 255) / 256 * 256;
-      nb = (int)((N + 127) / 128);
     }
     int64_t incl = bytes;
 #pragma unroll
@@ -1580,18 +1656,6 @@ batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int
     }
     if (t < L) table[t].packed_offset = base + incl - bytes;
     base += __shfl(incl, 63, 64);
-#pragma unroll
-    for (int c = 0; c < BATCH_CLASSES; c++) {
-      const int v = cls == c ? nb : 0;
-      int in = v;
-#pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const int up = __shfl_up(in, off, 64);
-        if (lane >= off) in += up;
-      }
-      if (cls == c) ws.tensor_class_off[t] = class_base[c] + in - v;
-      class_base[c] += __shfl(in, 63, 64);
-    }
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) {
@@ -1604,14 +1668,6 @@ batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int
     ws.hdr->ok = (!bad && base <= capacity) ? 1 : 0;
 #pragma unroll
     for (int k = 0; k < 4; k++) ws.hdr->tensors_at[k] = cnt[k];
-    ws.hdr->reserved[0] = ws.hdr->reserved[1] = 0;
-    int64_t run = 0;
-#pragma unroll
-    for (int c = 0; c < BATCH_CLASSES; c++) {
-      ws.hdr->class_count[c] = class_base[c];
-      ws.hdr->class_start[c] = run;
-      run += class_base[c];
-    }
   }
 }
 
@@ -1624,44 +1680,37 @@ __device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ t
   return lo;
 }
 
-// One thread per block of the grid: find its tensor, note it, and enter the block in its class's stretch of
-// the list.  Runs after the plan kernel on the same stream.
+// One thread per block of the grid: find its tensor and note it, so that a work kernel's block needs one load.
 __global__ void __launch_bounds__(256)
-batch_lists_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
-                   int64_t total_blocks, BatchWorkspace ws) {
+batch_blocks_kernel(const gact_batch_entry* __restrict__ table, int L, int64_t total_blocks, BatchWorkspace ws) {
   const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (g >= total_blocks) return;
-  const int t = batch_find(table, L, g);
-  int bt = bits[t];
-  if (!(bt == 1 || bt == 2 || bt == 4 || bt == 8)) bt = 8;   // as the plan counted it; the launch is void anyway
-  int dt = table[t].dtype;
-  if (dt < 0 || dt > 2) dt = 0;
-  const int cls = dt * 4 + width_index(bt);
-  const int local = (int)(g - table[t].first_block);
-  ws.block_tensor[g] = t;
-  ws.class_list[ws.hdr->class_start[cls] + ws.tensor_class_off[t] + local] = make_int2(t, local);
+  if (g < total_blocks) ws.block_tensor[g] = batch_find(table, L, g);
 }
 
-// Quantize, one launch per width and element type, so that every combination gets a kernel with its own
-// register allocation (176 registers at 1 bit float, 117 at 1 bit half, 34 at 8 bit half).  The workgroups
-// of a launch stride over the blocks of their class: the grid need not know how many there are.
-template <typename T, int BITS, int NOISE>
+// Quantize, one launch per element type over all blocks of the grid: the width of a block's tensor is read from
+// device memory and selects the code path (a row takes 8 groups whatever the width, so every path holds the same
+// amount of data in registers); blocks of tensors of another element type leave at once.
+template <typename T, int NOISE>
 __global__ void __launch_bounds__(256)
-quantize_batched_kernel(const gact_batch_entry* __restrict__ table, BatchWorkspace ws,
-                        uint8_t* __restrict__ packed_arena, uint8_t* __restrict__ scale_arena,
+quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits,
+                        BatchWorkspace ws, uint8_t* __restrict__ packed_arena, uint8_t* __restrict__ scale_arena,
                         uint8_t* __restrict__ min_arena) {
   if (ws.hdr->ok == 0) return;  // the plan did not fit the arena or held an invalid width
-  constexpr int CLS = Elem<T>::kDtype * 4 + (BITS == 1 ? 0 : BITS == 2 ? 1 : BITS == 4 ? 2 : 3);
-  const int64_t count = ws.hdr->class_count[CLS];
-  const int2* __restrict__ list = ws.class_list + ws.hdr->class_start[CLS];
-#pragma unroll 1
-  for (int64_t b = blockIdx.x; b < count; b += gridDim.x) {
-    const int2 e = list[b];
-    const gact_batch_entry ent = table[e.x];
-    const int64_t N = (ent.numel + GROUP - 1) / GROUP;
-    quantize_block128<T, BITS, NOISE>((const T*)ent.x, ent.numel, N, e.y, packed_arena + ent.packed_offset,
-                                      (typename Elem<T>::Stat*)(scale_arena + ent.stats_offset * 4),
-                                      (T*)(min_arena + ent.stats_offset * 4), ent.seed);
+  const int64_t block = xcd_tile<GACT_XCD_RUN_QB>(blockIdx.x, gridDim.x);
+  const int t = ws.block_tensor[block];
+  const gact_batch_entry ent = table[t];
+  if (ent.dtype != Elem<T>::kDtype) return;
+  const int64_t N = (ent.numel + GROUP - 1) / GROUP;
+  const int64_t lb = block - ent.first_block;
+  const T* x = (const T*)ent.x;
+  uint8_t* packed = packed_arena + ent.packed_offset;
+  typename Elem<T>::Stat* sc = (typename Elem<T>::Stat*)(scale_arena + ent.stats_offset * 4);
+  T* mn = (T*)(min_arena + ent.stats_offset * 4);
+  switch (bits[t]) {
+    case 1: quantize_block128<T, 1, NOISE>(x, ent.numel, N, lb, packed, sc, mn, ent.seed); break;
+    case 2: quantize_block128<T, 2, NOISE>(x, ent.numel, N, lb, packed, sc, mn, ent.seed); break;
+    case 4: quantize_block128<T, 4, NOISE>(x, ent.numel, N, lb, packed, sc, mn, ent.seed); break;
+    default: quantize_block128<T, 8, NOISE>(x, ent.numel, N, lb, packed, sc, mn, ent.seed); break;
   }
 }
 
@@ -1685,7 +1734,7 @@ dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int3
                           const uint8_t* __restrict__ scale_arena, const uint8_t* __restrict__ min_arena) {
   if (ws.hdr->ok == 0) return;
   // half a block is the single-tensor kernel's tile; same XCD-aware order (715 -> 709 us on 120 half tensors)
-  const uint32_t tile = xcd_tile<GACT_XCD_RUN_DQ>(blockIdx.x, gridDim.x);
+  const uint32_t tile = xcd_tile<GACT_XCD_RUN_DQB>(blockIdx.x, gridDim.x);
   const int64_t block = tile >> 1;
   const int half = tile & 1;
   const int t = ws.block_tensor[block];
@@ -1717,19 +1766,6 @@ inline void row_grid(int64_t rows, dim3* grid, dim3* block, int threads = 256) {
   const int rows_per_block = threads / 16;
   *grid = dim3((unsigned)((rows + rows_per_block - 1) / rows_per_block));
   *block = dim3(threads);
-}
-// Workgroup size of the quantize kernel.  A row's work grows with 8/bits groups; the long-running
-// low-width rows schedule better as single-wave workgroups (measured: float 2 bit 5.7 -> 6.2 TB/s,
-// 1 bit 5.4 -> 6.0 TB/s), the short high-width ones as four waves.
-#ifndef GACT_Q_BLOCK256_F32
-#define GACT_Q_BLOCK256_F32 8 /* width from which float rows run in four-wave workgroups */
-#endif
-#ifndef GACT_Q_BLOCK256_F16
-#define GACT_Q_BLOCK256_F16 4
-#endif
-inline int quantize_threads(int bits, size_t elem_size) {
-  const int from = elem_size == 4 ? GACT_Q_BLOCK256_F32 : GACT_Q_BLOCK256_F16;
-  return bits >= from ? 256 : 64;
 }
 inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8 / bits); }
 
@@ -1764,7 +1800,9 @@ int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, typen
                     int noise_mode,
                     SeedArg seed, const float* noise, hipStream_t stream) {
   dim3 grid, block;
-  row_grid(supergroups(N, BITS), &grid, &block, quantize_threads(BITS, sizeof(T)));
+  constexpr QGeom G = q_geom<T>(BITS);
+  const int sgr = noise_mode == GACT_NOISE_REF ? 1 : G.sgr;
+  row_grid((supergroups(N, BITS) + sgr - 1) / sgr, &grid, &block, G.threads);
   // the reference stream's one Philox block per byte makes the kernel instruction-bound: it wants every wave
   const unsigned lds = noise_mode == GACT_NOISE_REF ? 0u : quantize_lds_cap(sizeof(T), BITS, N);
   switch (noise_mode) {
@@ -1907,7 +1945,7 @@ const char* gact_strerror(int code) {
     case GACT_ESHAPE: return "unsupported shape";
     case GACT_ELAUNCH: return "HIP launch failed";
     case GACT_EBUDGET: return "bit budget unreachable: every tensor is already at 1 bit";
-    case GACT_ELIMIT: return "beyond the limit of the library's own workspace (4096 tensors, 262144 blocks of 128 groups)";
+    case GACT_ELIMIT: return "beyond the limit of the library's own workspace (262144 blocks of 128 groups)";
   }
   return "unknown error";
 }
@@ -2104,39 +2142,27 @@ int64_t gact_batch_workspace_bytes(int64_t L, int64_t total_blocks) {
 namespace {
 int batch_plan_on(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks, int64_t capacity,
                   void* workspace, hipStream_t s) {
-  const BatchWorkspace ws = batch_workspace(workspace, L, total_blocks);
+  const BatchWorkspace ws = batch_workspace(workspace);
   hipLaunchKernelGGL(batch_plan_kernel, dim3(1), dim3(64), 0, s, table, bits, (int)L, capacity, ws);
   if (total_blocks > 0)
-    hipLaunchKernelGGL(batch_lists_kernel, dim3((unsigned)((total_blocks + 255) / 256)), dim3(256), 0, s, table, bits, (int)L,
+    hipLaunchKernelGGL(batch_blocks_kernel, dim3((unsigned)((total_blocks + 255) / 256)), dim3(256), 0, s, table, (int)L,
                        total_blocks, ws);
   return launch_status();
 }
 
-int quantize_batched_on(const gact_batch_entry* table, int64_t L, int64_t total_blocks, int noise_mode, int dtypes,
-                        void* workspace, void* packed_arena, void* scale_arena, void* min_arena, hipStream_t s) {
-  const BatchWorkspace ws = batch_workspace(workspace, L, total_blocks);
-  // the widths live on the device, so a launch cannot be sized to its class: a quarter of the blocks (all of
-  // them when there are few), striding over the class's list, keeps the chip full and the empty classes cheap
-  int64_t g = total_blocks / 4;
-  if (g < 8192) g = total_blocks < 8192 ? total_blocks : 8192;
-  const dim3 grid((unsigned)g), block(256);
-#define GACT_LAUNCH_QB(T, B, M)                                                                               \
-  hipLaunchKernelGGL((quantize_batched_kernel<T, B, M>), grid, block, 0, s, table, ws, (uint8_t*)packed_arena, \
+int quantize_batched_on(const gact_batch_entry* table, const int32_t* bits, int64_t total_blocks, int noise_mode,
+                        int dtypes, void* workspace, void* packed_arena, void* scale_arena, void* min_arena,
+                        hipStream_t s) {
+  const BatchWorkspace ws = batch_workspace(workspace);
+  const dim3 grid((unsigned)total_blocks), block(256);
+#define GACT_LAUNCH_QB(T, M)                                                                                  \
+  hipLaunchKernelGGL((quantize_batched_kernel<T, M>), grid, block, 0, s, table, bits, ws, (uint8_t*)packed_arena, \
                      (uint8_t*)scale_arena, (uint8_t*)min_arena)
 #define GACT_LAUNCH_QB_ALL(M)                                                                                 \
   do {                                                                                                        \
-    if (dtypes & GACT_DTYPES_F32) {                                                                           \
-      GACT_LAUNCH_QB(float, 1, M); GACT_LAUNCH_QB(float, 2, M); GACT_LAUNCH_QB(float, 4, M);                  \
-      GACT_LAUNCH_QB(float, 8, M);                                                                            \
-    }                                                                                                         \
-    if (dtypes & GACT_DTYPES_F16) {                                                                           \
-      GACT_LAUNCH_QB(f16, 1, M); GACT_LAUNCH_QB(f16, 2, M); GACT_LAUNCH_QB(f16, 4, M);                        \
-      GACT_LAUNCH_QB(f16, 8, M);                                                                              \
-    }                                                                                                         \
-    if (dtypes & GACT_DTYPES_BF16) {                                                                          \
-      GACT_LAUNCH_QB(bf16, 1, M); GACT_LAUNCH_QB(bf16, 2, M); GACT_LAUNCH_QB(bf16, 4, M);                     \
-      GACT_LAUNCH_QB(bf16, 8, M);                                                                             \
-    }                                                                                                         \
+    if (dtypes & GACT_DTYPES_F32) GACT_LAUNCH_QB(float, M);                                                   \
+    if (dtypes & GACT_DTYPES_F16) GACT_LAUNCH_QB(f16, M);                                                     \
+    if (dtypes & GACT_DTYPES_BF16) GACT_LAUNCH_QB(bf16, M);                                                   \
   } while (0)
   switch (noise_mode) {
     case GACT_NOISE_CONST: GACT_LAUNCH_QB_ALL(GACT_NOISE_CONST); break;
@@ -2173,7 +2199,7 @@ int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, in
   if (L == 0 || total_blocks == 0) return GACT_OK;
   if (!table || !bits || !workspace || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena) || !aligned16(workspace)) return GACT_EALIGN;
-  return quantize_batched_on(table, L, total_blocks, noise_mode, dtypes, const_cast<void*>(workspace), packed_arena,
+  return quantize_batched_on(table, bits, total_blocks, noise_mode, dtypes, const_cast<void*>(workspace), packed_arena,
                              scale_arena, min_arena, (hipStream_t)stream);
 }
 
@@ -2186,7 +2212,7 @@ int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, 
   if (!aligned16(packed_arena) || !aligned16(workspace)) return GACT_EALIGN;
   const dim3 grid((unsigned)(2 * total_blocks)), block(256);
   hipLaunchKernelGGL(dequantize_batched_kernel, grid, block, 0, (hipStream_t)stream, table, bits,
-                     batch_workspace(const_cast<void*>(workspace), L, total_blocks), (const uint8_t*)packed_arena,
+                     batch_workspace(const_cast<void*>(workspace)), (const uint8_t*)packed_arena,
                      (const uint8_t*)scale_arena, (const uint8_t*)min_arena);
   return launch_status();
 }
@@ -2198,9 +2224,8 @@ int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, 
 // handle) and that pointer is what the kernels get.  Calls on one GPU share the array: they must not overlap.
 // Nothing in it has to start at zero - the plan kernels write every field the work kernels read.
 // ------------------------------------------------------------------------------------------------
-#define GACT_STATIC_MAX_TENSORS 4096
 #define GACT_STATIC_MAX_BLOCKS 262144
-#define GACT_STATIC_WORKSPACE_BYTES (256 + GACT_STATIC_MAX_TENSORS * 4 + GACT_STATIC_MAX_BLOCKS * 12)
+#define GACT_STATIC_WORKSPACE_BYTES (256 + GACT_STATIC_MAX_BLOCKS * 4)
 #define GACT_MAX_DEVICES 64
 static __device__ __align__(256) __attribute__((used)) unsigned char scratch[GACT_STATIC_WORKSPACE_BYTES];
 
@@ -2229,9 +2254,7 @@ int gact_quantize_batched_static(gact_batch_entry* table, const int32_t* bits, i
   if (noise_mode != GACT_NOISE_CONST && noise_mode != GACT_NOISE_REF && noise_mode != GACT_NOISE_FAST) return GACT_EINVAL;
   if (dtypes < 0 || dtypes > GACT_DTYPES_ALL) return GACT_EINVAL;
   if (dtypes == 0) dtypes = GACT_DTYPES_ALL;
-  if (L > GACT_STATIC_MAX_TENSORS || total_blocks > GACT_STATIC_MAX_BLOCKS) return GACT_ELIMIT;
-  static_assert(GACT_STATIC_WORKSPACE_BYTES >= 256 + GACT_STATIC_MAX_TENSORS * 4 + GACT_STATIC_MAX_BLOCKS * 4 + GACT_STATIC_MAX_BLOCKS * 8,
-                "the array holds the workspace of the largest table");
+  if (total_blocks > GACT_STATIC_MAX_BLOCKS) return GACT_ELIMIT;
   if (L == 0 || total_blocks == 0) return GACT_OK;
   if (!table || !bits || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena)) return GACT_EALIGN;
@@ -2241,7 +2264,7 @@ int gact_quantize_batched_static(gact_batch_entry* table, const int32_t* bits, i
   hipStream_t s = (hipStream_t)stream;
   const int planned = batch_plan_on(table, bits, L, total_blocks, capacity, ws, s);
   if (planned != GACT_OK) return planned;
-  return quantize_batched_on(table, L, total_blocks, noise_mode, dtypes, ws, packed_arena, scale_arena, min_arena, s);
+  return quantize_batched_on(table, bits, total_blocks, noise_mode, dtypes, ws, packed_arena, scale_arena, min_arena, s);
 }
 
 }  // extern "C"
