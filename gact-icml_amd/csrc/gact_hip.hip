@@ -1600,9 +1600,8 @@ calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, cons
 // Batched launch over a table of tensors with device-resident bits.
 // ------------------------------------------------------------------------------------------------
 // The workspace of a batched launch (device memory the caller brings, or the library's static array):
-//   BatchHeader                 what the plan found
-//   BatchBlock[total_blocks]    one self-contained record per block of the grid: a work kernel's block reads
-//                               its record with one scalar load and needs nothing else before its data
+//   BatchHeader                      what the plan found
+//   int32 block_tensor[total_blocks] tensor of every block of the grid
 struct BatchHeader {
   int64_t need;            // arena bytes the table needs
   int64_t ok;              // 1: every width and element type valid and need <= capacity
@@ -1610,30 +1609,18 @@ struct BatchHeader {
   int64_t reserved[26];
 };
 static_assert(sizeof(BatchHeader) == 256, "the header is 32 int64");
-struct BatchBlock {
-  const void* x;          // the tensor's activation
-  int64_t numel;
-  int64_t packed_offset;  // the tensor's codes in the packed arena
-  int64_t stats_offset;   // the tensor's rows in the scale / min arenas
-  uint64_t seed;
-  int32_t lb;             // this block within its tensor
-  int32_t bits;           // 1, 2, 4, 8; 0: the launch is void (the plan failed), do nothing
-  int32_t dtype;
-  int32_t pad[3];
-};
-static_assert(sizeof(BatchBlock) == 64, "a block record is one 64-byte line");
 struct BatchWorkspace {
   BatchHeader* hdr;
-  BatchBlock* blocks;
+  int32_t* block_tensor;
 };
 __host__ __device__ inline int64_t batch_workspace_need(int64_t L, int64_t total_blocks) {
   (void)L;
-  return (int64_t)sizeof(BatchHeader) + total_blocks * (int64_t)sizeof(BatchBlock);
+  return (int64_t)sizeof(BatchHeader) + (total_blocks + 3) / 4 * 16;
 }
 __host__ __device__ inline BatchWorkspace batch_workspace(void* base) {
   BatchWorkspace w;
   w.hdr = (BatchHeader*)base;
-  w.blocks = (BatchBlock*)((uint8_t*)base + sizeof(BatchHeader));
+  w.block_tensor = (int32_t*)((uint8_t*)base + sizeof(BatchHeader));
   return w;
 }
 __device__ __forceinline__ int width_index(int bits) { return bits == 1 ? 0 : bits == 2 ? 1 : bits == 4 ? 2 : 3; }
@@ -1693,81 +1680,74 @@ __device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ t
   return lo;
 }
 
-// One thread per block of the grid: find its tensor and write the block's record.  Runs after the plan kernel on
-// the same stream (it copies the offsets and the verdict the plan left).
+// One thread per block of the grid: find its tensor and note it, so that a work kernel's block needs one load.
 __global__ void __launch_bounds__(256)
-batch_blocks_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits, int L,
-                    int64_t total_blocks, BatchWorkspace ws) {
+batch_blocks_kernel(const gact_batch_entry* __restrict__ table, int L, int64_t total_blocks, BatchWorkspace ws) {
   const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (g >= total_blocks) return;
-  const int t = batch_find(table, L, g);
-  const gact_batch_entry ent = table[t];
-  BatchBlock rec;
-  rec.x = ent.x;
-  rec.numel = ent.numel;
-  rec.packed_offset = ent.packed_offset;
-  rec.stats_offset = ent.stats_offset;
-  rec.seed = ent.seed;
-  rec.lb = (int32_t)(g - ent.first_block);
-  rec.bits = ws.hdr->ok ? bits[t] : 0;
-  rec.dtype = ent.dtype;
-  rec.pad[0] = rec.pad[1] = rec.pad[2] = 0;
-  ws.blocks[g] = rec;
+  if (g < total_blocks) ws.block_tensor[g] = batch_find(table, L, g);
 }
 
-// Quantize, one launch per element type over all blocks of the grid: the width in a block's record selects the
-// code path (a row takes 8 groups whatever the width, so every path holds the same amount of data in registers);
-// blocks of tensors of another element type leave at once.
+// Quantize, one launch per element type over all blocks of the grid: the width of a block's tensor is read from
+// device memory and selects the code path (a row takes 8 groups whatever the width, so every path holds the same
+// amount of data in registers); blocks of tensors of another element type leave at once.
 template <typename T, int NOISE>
 __global__ void __launch_bounds__(256)
-quantize_batched_kernel(BatchWorkspace ws, uint8_t* __restrict__ packed_arena, uint8_t* __restrict__ scale_arena,
+quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits,
+                        BatchWorkspace ws, uint8_t* __restrict__ packed_arena, uint8_t* __restrict__ scale_arena,
                         uint8_t* __restrict__ min_arena) {
-  const BatchBlock rec = ws.blocks[xcd_tile<GACT_XCD_RUN_QB>(blockIdx.x, gridDim.x)];
-  if (rec.dtype != Elem<T>::kDtype) return;
-  const int64_t N = (rec.numel + GROUP - 1) / GROUP;
-  const T* x = (const T*)rec.x;
-  uint8_t* packed = packed_arena + rec.packed_offset;
-  typename Elem<T>::Stat* sc = (typename Elem<T>::Stat*)(scale_arena + rec.stats_offset * 4);
-  T* mn = (T*)(min_arena + rec.stats_offset * 4);
-  switch (rec.bits) {
-    case 1: quantize_block128<T, 1, NOISE>(x, rec.numel, N, rec.lb, packed, sc, mn, rec.seed); break;
-    case 2: quantize_block128<T, 2, NOISE>(x, rec.numel, N, rec.lb, packed, sc, mn, rec.seed); break;
-    case 4: quantize_block128<T, 4, NOISE>(x, rec.numel, N, rec.lb, packed, sc, mn, rec.seed); break;
-    case 8: quantize_block128<T, 8, NOISE>(x, rec.numel, N, rec.lb, packed, sc, mn, rec.seed); break;
-    default: break;   // 0: the plan did not fit the arena or held an invalid width
+  if (ws.hdr->ok == 0) return;  // the plan did not fit the arena or held an invalid width
+  const int64_t block = xcd_tile<GACT_XCD_RUN_QB>(blockIdx.x, gridDim.x);
+  const int t = ws.block_tensor[block];
+  const gact_batch_entry ent = table[t];
+  if (ent.dtype != Elem<T>::kDtype) return;
+  const int64_t N = (ent.numel + GROUP - 1) / GROUP;
+  const int64_t lb = block - ent.first_block;
+  const T* x = (const T*)ent.x;
+  uint8_t* packed = packed_arena + ent.packed_offset;
+  typename Elem<T>::Stat* sc = (typename Elem<T>::Stat*)(scale_arena + ent.stats_offset * 4);
+  T* mn = (T*)(min_arena + ent.stats_offset * 4);
+  switch (bits[t]) {
+    case 1: quantize_block128<T, 1, NOISE>(x, ent.numel, N, lb, packed, sc, mn, ent.seed); break;
+    case 2: quantize_block128<T, 2, NOISE>(x, ent.numel, N, lb, packed, sc, mn, ent.seed); break;
+    case 4: quantize_block128<T, 4, NOISE>(x, ent.numel, N, lb, packed, sc, mn, ent.seed); break;
+    default: quantize_block128<T, 8, NOISE>(x, ent.numel, N, lb, packed, sc, mn, ent.seed); break;
   }
 }
 
-// Dequantize, one launch for all widths and element types (every path fits 60 registers), so no workgroup is
-// launched only to leave.
+// Dequantize, one launch for all widths (every width fits 60 registers): the width of a block's tensor is read
+// from device memory and selects the code path, so no workgroup is launched only to leave.
 template <int BITS>
-__device__ __forceinline__ void dequantize_batched_block(const BatchBlock& rec, int half, const uint8_t* packed,
-                                                         const uint8_t* sc, const uint8_t* mn) {
-  const int64_t N = (rec.numel + GROUP - 1) / GROUP;
-  if (rec.dtype == GACT_F32)
-    dequantize_block128<float, BITS>(packed, (const float*)sc, (const float*)mn, rec.numel, N, rec.lb, half, (float*)rec.x);
-  else if (rec.dtype == GACT_F16)
-    dequantize_block128<f16, BITS>(packed, (const f16*)sc, (const f16*)mn, rec.numel, N, rec.lb, half, (f16*)rec.x);
+__device__ __forceinline__ void dequantize_batched_block(const gact_batch_entry& ent, int64_t lb, int half,
+                                                         const uint8_t* packed, const uint8_t* sc, const uint8_t* mn) {
+  const int64_t N = (ent.numel + GROUP - 1) / GROUP;
+  if (ent.dtype == GACT_F32)
+    dequantize_block128<float, BITS>(packed, (const float*)sc, (const float*)mn, ent.numel, N, lb, half, (float*)ent.x);
+  else if (ent.dtype == GACT_F16)
+    dequantize_block128<f16, BITS>(packed, (const f16*)sc, (const f16*)mn, ent.numel, N, lb, half, (f16*)ent.x);
   else
-    dequantize_block128<bf16, BITS>(packed, (const float*)sc, (const bf16*)mn, rec.numel, N, rec.lb, half, (bf16*)rec.x);
+    dequantize_block128<bf16, BITS>(packed, (const float*)sc, (const bf16*)mn, ent.numel, N, lb, half, (bf16*)ent.x);
 }
 // grid: two workgroups per block of 128 groups
 __global__ void __launch_bounds__(256)
-dequantize_batched_kernel(BatchWorkspace ws, const uint8_t* __restrict__ packed_arena,
+dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits,
+                          BatchWorkspace ws, const uint8_t* __restrict__ packed_arena,
                           const uint8_t* __restrict__ scale_arena, const uint8_t* __restrict__ min_arena) {
+  if (ws.hdr->ok == 0) return;
   // half a block is the single-tensor kernel's tile; same XCD-aware order (715 -> 709 us on 120 half tensors)
   const uint32_t tile = xcd_tile<GACT_XCD_RUN_DQB>(blockIdx.x, gridDim.x);
-  const BatchBlock rec = ws.blocks[tile >> 1];
+  const int64_t block = tile >> 1;
   const int half = tile & 1;
-  const uint8_t* packed = packed_arena + rec.packed_offset;
-  const uint8_t* sc = scale_arena + rec.stats_offset * 4;
-  const uint8_t* mn = min_arena + rec.stats_offset * 4;
-  switch (rec.bits) {
-    case 1: dequantize_batched_block<1>(rec, half, packed, sc, mn); break;
-    case 2: dequantize_batched_block<2>(rec, half, packed, sc, mn); break;
-    case 4: dequantize_batched_block<4>(rec, half, packed, sc, mn); break;
-    case 8: dequantize_batched_block<8>(rec, half, packed, sc, mn); break;
-    default: break;   // 0: a void launch
+  const int t = ws.block_tensor[block];
+  const gact_batch_entry ent = table[t];
+  const int64_t lb = block - ent.first_block;
+  const uint8_t* packed = packed_arena + ent.packed_offset;
+  const uint8_t* sc = scale_arena + ent.stats_offset * 4;
+  const uint8_t* mn = min_arena + ent.stats_offset * 4;
+  switch (bits[t]) {
+    case 1: dequantize_batched_block<1>(ent, lb, half, packed, sc, mn); break;
+    case 2: dequantize_batched_block<2>(ent, lb, half, packed, sc, mn); break;
+    case 4: dequantize_batched_block<4>(ent, lb, half, packed, sc, mn); break;
+    default: dequantize_batched_block<8>(ent, lb, half, packed, sc, mn); break;
   }
 }
 
@@ -1965,7 +1945,7 @@ const char* gact_strerror(int code) {
     case GACT_ESHAPE: return "unsupported shape";
     case GACT_ELAUNCH: return "HIP launch failed";
     case GACT_EBUDGET: return "bit budget unreachable: every tensor is already at 1 bit";
-    case GACT_ELIMIT: return "beyond the limit of the library's own workspace (65536 blocks of 128 groups)";
+    case GACT_ELIMIT: return "beyond the limit of the library's own workspace (262144 blocks of 128 groups)";
   }
   return "unknown error";
 }
@@ -2165,17 +2145,18 @@ int batch_plan_on(gact_batch_entry* table, const int32_t* bits, int64_t L, int64
   const BatchWorkspace ws = batch_workspace(workspace);
   hipLaunchKernelGGL(batch_plan_kernel, dim3(1), dim3(64), 0, s, table, bits, (int)L, capacity, ws);
   if (total_blocks > 0)
-    hipLaunchKernelGGL(batch_blocks_kernel, dim3((unsigned)((total_blocks + 255) / 256)), dim3(256), 0, s, table, bits,
-                       (int)L, total_blocks, ws);
+    hipLaunchKernelGGL(batch_blocks_kernel, dim3((unsigned)((total_blocks + 255) / 256)), dim3(256), 0, s, table, (int)L,
+                       total_blocks, ws);
   return launch_status();
 }
 
-int quantize_batched_on(int64_t total_blocks, int noise_mode, int dtypes, void* workspace, void* packed_arena,
-                        void* scale_arena, void* min_arena, hipStream_t s) {
+int quantize_batched_on(const gact_batch_entry* table, const int32_t* bits, int64_t total_blocks, int noise_mode,
+                        int dtypes, void* workspace, void* packed_arena, void* scale_arena, void* min_arena,
+                        hipStream_t s) {
   const BatchWorkspace ws = batch_workspace(workspace);
   const dim3 grid((unsigned)total_blocks), block(256);
 #define GACT_LAUNCH_QB(T, M)                                                                                  \
-  hipLaunchKernelGGL((quantize_batched_kernel<T, M>), grid, block, 0, s, ws, (uint8_t*)packed_arena,          \
+  hipLaunchKernelGGL((quantize_batched_kernel<T, M>), grid, block, 0, s, table, bits, ws, (uint8_t*)packed_arena, \
                      (uint8_t*)scale_arena, (uint8_t*)min_arena)
 #define GACT_LAUNCH_QB_ALL(M)                                                                                 \
   do {                                                                                                        \
@@ -2218,8 +2199,8 @@ int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, in
   if (L == 0 || total_blocks == 0) return GACT_OK;
   if (!table || !bits || !workspace || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena) || !aligned16(workspace)) return GACT_EALIGN;
-  return quantize_batched_on(total_blocks, noise_mode, dtypes, const_cast<void*>(workspace), packed_arena, scale_arena,
-                             min_arena, (hipStream_t)stream);
+  return quantize_batched_on(table, bits, total_blocks, noise_mode, dtypes, const_cast<void*>(workspace), packed_arena,
+                             scale_arena, min_arena, (hipStream_t)stream);
 }
 
 int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
@@ -2230,10 +2211,7 @@ int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, 
   if (!table || !bits || !workspace || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena) || !aligned16(workspace)) return GACT_EALIGN;
   const dim3 grid((unsigned)(2 * total_blocks)), block(256);
-#ifndef GACT_DQB_LDS
-#define GACT_DQB_LDS 0
-#endif
-  hipLaunchKernelGGL(dequantize_batched_kernel, grid, block, GACT_DQB_LDS, (hipStream_t)stream,
+  hipLaunchKernelGGL(dequantize_batched_kernel, grid, block, 0, (hipStream_t)stream, table, bits,
                      batch_workspace(const_cast<void*>(workspace)), (const uint8_t*)packed_arena,
                      (const uint8_t*)scale_arena, (const uint8_t*)min_arena);
   return launch_status();
@@ -2246,8 +2224,8 @@ int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, 
 // handle) and that pointer is what the kernels get.  Calls on one GPU share the array: they must not overlap.
 // Nothing in it has to start at zero - the plan kernels write every field the work kernels read.
 // ------------------------------------------------------------------------------------------------
-#define GACT_STATIC_MAX_BLOCKS 65536
-#define GACT_STATIC_WORKSPACE_BYTES (256 + GACT_STATIC_MAX_BLOCKS * 64)
+#define GACT_STATIC_MAX_BLOCKS 262144
+#define GACT_STATIC_WORKSPACE_BYTES (256 + GACT_STATIC_MAX_BLOCKS * 4)
 #define GACT_MAX_DEVICES 64
 static __device__ __align__(256) __attribute__((used)) unsigned char scratch[GACT_STATIC_WORKSPACE_BYTES];
 
@@ -2286,7 +2264,7 @@ int gact_quantize_batched_static(gact_batch_entry* table, const int32_t* bits, i
   hipStream_t s = (hipStream_t)stream;
   const int planned = batch_plan_on(table, bits, L, total_blocks, capacity, ws, s);
   if (planned != GACT_OK) return planned;
-  return quantize_batched_on(total_blocks, noise_mode, dtypes, ws, packed_arena, scale_arena, min_arena, s);
+  return quantize_batched_on(table, bits, total_blocks, noise_mode, dtypes, ws, packed_arena, scale_arena, min_arena, s);
 }
 
 }  // extern "C"

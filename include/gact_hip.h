@@ -126,8 +126,7 @@ int64_t gact_batch_workspace_bytes(int64_t L, int64_t total_blocks);
 /* Plan a batched launch from device-resident bits: fills packed_offset of every table entry (256-byte
  * aligned, in table order) and the workspace - a header of 32 int64 ([0] the arena bytes the table needs,
  * [1] 1 when every bits[i] is in {1,2,4,8}, every dtype is known and [0] <= capacity, else 0: the batched
- * kernels then do nothing, [2..5] the number of tensors at width 1, 2, 4, 8) and one 64-byte record per block
- * (the block's tensor, offsets, seed, width), which is all a work kernel's block reads before its data.
+ * kernels then do nothing, [2..5] the number of tensors at width 1, 2, 4, 8) and the tensor of every block.
  * Two small kernels; nothing is read back.  No counterpart in the reference. */
 int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
                     int64_t capacity, void* workspace, void* stream);
@@ -139,8 +138,7 @@ int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int
  * the rows stay 32-byte aligned).  Results equal a loop of
  * gact_quantize / gact_dequantize over the tensors (gact/gact/quantizer.py:95-142 drives the reference
  * one tensor at a time).  `workspace` is what gact_batch_plan filled for the same table, bits, L and
- * total_blocks: the work kernels read the records it holds, so plan again whenever the table or the widths
- * change (another set of output tensors included).  `dtypes` says which element types
+ * total_blocks.  `dtypes` says which element types
  * occur in the table, which the host that built it knows: bit 0 float, bit 1 half, bit 2 bfloat16 (GACT_DTYPES_*); quantize
  * launches only the kernels of those types, so a tensor whose type is missing from the mask is left unquantized. */
 #define GACT_DTYPES_F32 1
@@ -155,12 +153,12 @@ int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, 
                             const void* scale_arena, const void* min_arena, void* stream);
 
 /* gact_batch_plan followed by gact_quantize_batched, with the workspace in a device array that is part of
- * the library (4 MB per GPU the library runs on, held until the process ends) instead of memory the
+ * the library (1 MB per GPU the library runs on, held until the process ends) instead of memory the
  * caller brings: nothing is allocated, by the library or on its behalf.  No counterpart in the reference; it
  * is for callers that cannot allocate - code under HIP graph capture, tight serving loops, harnesses that
  * forbid it.  Same results as the two calls it stands for (packed_offset of every table entry is filled, the
  * arenas are written); the plan's verdict stays in the library's array, so size the arena for the worst case
- * or check the widths beforehand.  Limit: total_blocks <= 65536 (8.4 M groups, 2.1 G elements),
+ * or check the widths beforehand.  Limit: total_blocks <= 262144 (33.5 M groups, 8.6 G elements),
  * GACT_ELIMIT beyond.  All calls on one GPU share the array: calls that overlap on one GPU (two streams, two
  * threads) race, the caller serialises them.  The first call on a GPU looks the array's address up; make it
  * outside a stream capture.  Dequantize with gact_batch_plan + gact_dequantize_batched as usual. */

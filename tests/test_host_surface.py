@@ -75,9 +75,9 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     assert L.gact_quantize_batched(16, 16, 3, 3, 0, 3, 8, 16, 16, 16, None) == -2                # misaligned workspace
     assert L.gact_batch_plan(16, 16, 3, 3, -1, 16, None) == -1                                   # negative capacity
     assert L.gact_batch_plan(16, 16, 3, 3, 100, None, None) == -1                                # no workspace
-    # header (32 int64) + one 64-byte record per block
-    assert L.gact_batch_workspace_bytes(3, 5) == 256 + 5 * 64
-    assert L.gact_quantize_batched_static(16, 16, 10, 65537, 1 << 20, 3, 0, 16, 16, 16, None) == -6   # beyond its array
+    # header (32 int64) + one int32 per block, in whole 16-byte pieces
+    assert L.gact_batch_workspace_bytes(3, 5) == 256 + 2 * 16
+    assert L.gact_quantize_batched_static(16, 16, 10, 262145, 1 << 20, 3, 0, 16, 16, 16, None) == -6   # beyond its array
     assert L.gact_batch_workspace_bytes(-1, 5) == -1
     assert L.gact_quantize(16, 3, 256, 4, 0, 0, None, 16, 16, 16, None, None) == -1               # element type
     assert L.gact_quantize(0, 2, 256, 4, 0, 0, None, 16, 16, 16, None, None) == -1                # bfloat16, null data

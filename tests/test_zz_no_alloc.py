@@ -69,6 +69,6 @@ def test_static_workspace_matches_caller_workspace_twice_in_a_row():
 def test_static_workspace_limits():
     lib = _abi.lib()
     # beyond the array: refused before anything is launched (the pointers are never touched)
-    assert lib.gact_quantize_batched_static(16, 16, 10, 65537, 1 << 20, 3, 0, 16, 16, 16, None) == -6
+    assert lib.gact_quantize_batched_static(16, 16, 10, 262145, 1 << 20, 3, 0, 16, 16, 16, None) == -6
     assert lib.gact_quantize_batched_static(16, 16, 10, 1 << 29, 1 << 20, 3, 0, 16, 16, 16, None) == -6
     assert b"limit" in lib.gact_strerror(-6)
