@@ -1625,11 +1625,28 @@ __host__ __device__ inline BatchWorkspace batch_workspace(void* base) {
 }
 __device__ __forceinline__ int width_index(int bits) { return bits == 1 ? 0 : bits == 2 ? 1 : bits == 4 ? 2 : 3; }
 
-// One wave: lane l sizes tensors l, l+64, ...; the running packed-arena offset is carried across rounds of 64
-// with a wave-wide inclusive scan.
-__global__ void __launch_bounds__(64)
-batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int L, int64_t capacity,
-                  BatchWorkspace ws) {
+__device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ table, int L, int64_t block) {
+  int lo = 0, hi = L - 1;  // last entry with first_block <= block
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (table[mid].first_block <= block) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+// The plan, one launch.  Workgroup 0 (its first wave): lane l sizes tensors l, l+64, ...; the running packed-arena
+// offset is carried across rounds of 64 with a wave-wide inclusive scan.  The other workgroups, one thread per
+// block of the grid: find the block's tensor and note it, so that a work kernel's block needs one load for it
+// (this part depends on the geometry only, not on the widths).
+__global__ void __launch_bounds__(256)
+batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int L, int64_t total_blocks,
+                  int64_t capacity, BatchWorkspace ws) {
+  if (blockIdx.x > 0) {
+    const int64_t g = (int64_t)(blockIdx.x - 1) * blockDim.x + threadIdx.x;
+    if (g < total_blocks) ws.block_tensor[g] = batch_find(table, L, g);
+    return;
+  }
+  if (threadIdx.x >= 64) return;
   const int lane = threadIdx.x;
   int64_t base = 0;
   int bad = 0;
@@ -1669,22 +1686,6 @@ batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int
 #pragma unroll
     for (int k = 0; k < 4; k++) ws.hdr->tensors_at[k] = cnt[k];
   }
-}
-
-__device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ table, int L, int64_t block) {
-  int lo = 0, hi = L - 1;  // last entry with first_block <= block
-  while (lo < hi) {
-    const int mid = (lo + hi + 1) >> 1;
-    if (table[mid].first_block <= block) lo = mid; else hi = mid - 1;
-  }
-  return lo;
-}
-
-// One thread per block of the grid: find its tensor and note it, so that a work kernel's block needs one load.
-__global__ void __launch_bounds__(256)
-batch_blocks_kernel(const gact_batch_entry* __restrict__ table, int L, int64_t total_blocks, BatchWorkspace ws) {
-  const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (g < total_blocks) ws.block_tensor[g] = batch_find(table, L, g);
 }
 
 // Quantize, one launch per element type over all blocks of the grid: the width of a block's tensor is read from
@@ -2143,10 +2144,8 @@ namespace {
 int batch_plan_on(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks, int64_t capacity,
                   void* workspace, hipStream_t s) {
   const BatchWorkspace ws = batch_workspace(workspace);
-  hipLaunchKernelGGL(batch_plan_kernel, dim3(1), dim3(64), 0, s, table, bits, (int)L, capacity, ws);
-  if (total_blocks > 0)
-    hipLaunchKernelGGL(batch_blocks_kernel, dim3((unsigned)((total_blocks + 255) / 256)), dim3(256), 0, s, table, (int)L,
-                       total_blocks, ws);
+  hipLaunchKernelGGL(batch_plan_kernel, dim3((unsigned)(1 + (total_blocks + 255) / 256)), dim3(256), 0, s, table, bits, (int)L,
+                     total_blocks, capacity, ws);
   return launch_status();
 }
 

@@ -127,7 +127,7 @@ int64_t gact_batch_workspace_bytes(int64_t L, int64_t total_blocks);
  * aligned, in table order) and the workspace - a header of 32 int64 ([0] the arena bytes the table needs,
  * [1] 1 when every bits[i] is in {1,2,4,8}, every dtype is known and [0] <= capacity, else 0: the batched
  * kernels then do nothing, [2..5] the number of tensors at width 1, 2, 4, 8) and the tensor of every block.
- * Two small kernels; nothing is read back.  No counterpart in the reference. */
+ * One small launch; nothing is read back.  No counterpart in the reference. */
 int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
                     int64_t capacity, void* workspace, void* stream);
 
