@@ -1788,8 +1788,14 @@ inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8
 constexpr int64_t kCapFromGroups = GACT_CAP_FROM_GROUPS;
 inline unsigned dequantize_lds_cap(size_t elem_size, int bits, int64_t N) {
   if (N < kCapFromGroups) return 0u;
-  if (elem_size == 4) return 53000u;
-  return bits == 8 ? 40000u : 0u;
+#ifndef GACT_DQ_LDS_F32
+#define GACT_DQ_LDS_F32 53000u
+#endif
+#ifndef GACT_DQ_LDS_F16_LOW
+#define GACT_DQ_LDS_F16_LOW 0u
+#endif
+  if (elem_size == 4) return GACT_DQ_LDS_F32;
+  return bits == 8 ? 40000u : GACT_DQ_LDS_F16_LOW;
 }
 inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
   if (elem_size != 4 || N < kCapFromGroups) return 0u;

@@ -41,7 +41,8 @@ class QuantizationConfig:
         self.device_seed = False
 
         # ---- stochastic-rounding noise (not in the reference) ----
-        # "fast":          one Philox4x32-10 block per 8 elements, 16-bit uniforms
+        # "fast":          one Philox4x32-7 block per 16 elements (8 draws of 16 bits, each used once as u and once,
+        #                  half a group further on, as 1 - u)
         # "reference":     the reference's stream (one Philox state per output byte, cuRAND uniform map)
         # "deterministic": u = 0.5 everywhere, i.e. round to nearest
         self.rng_stream = "fast"
