@@ -756,9 +756,10 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
 }
 
 // ------------------------------------------------------------------------------------------------
-// Dequantize a unit of 8 consecutive groups (BITS super-groups).  A lane owns the W = 16/sizeof(T)
-// columns W*l .. W*l+W-1 of every group (one 16-byte store per group), so 256/W lanes cover a group:
-// a whole wave per unit for float, half a wave for half.  All code words are loaded first, then the 8
+// Dequantize a unit: G = SGS * (8/BITS) / PARTS consecutive groups - SGS whole super-groups, or (PARTS > 1, SGS = 1)
+// one of PARTS equal parts of a super-group, the code words of which its other units load as well.  A lane owns the
+// W = 16/sizeof(T) columns W*l .. W*l+W-1 of every group (one 16-byte store per group), so 256/W lanes cover a
+// group: a whole wave per unit for float, half a wave for half.  All code words are loaded first, then the
 // groups are written, each store instruction covering whole groups contiguously.
 // The values follow quantization_cuda_kernel.cu:149-177: T(code) / scale with a real division, + min.
 // 1, 2 and 4 bit tabulate the 2^BITS values of a group once and look them up; 8 bit computes
@@ -778,7 +779,7 @@ __device__ __forceinline__ float row_bcast_at(float v, int g) {
   }
 }
 
-template <typename T, int BITS, int SGS>
+template <typename T, int BITS, int SGS, int PARTS = 1>
 __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ packed,
                                                 const typename Elem<T>::Stat* __restrict__ scale,
                                                 const T* __restrict__ mn, int64_t numel, int64_t N, int64_t unit,
@@ -786,11 +787,14 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
   typedef typename Elem<T>::Stat Stat;
   constexpr int WPT = 8 / BITS;
   constexpr int W = Elem<T>::kDqWidth;
-  constexpr int G = SGS * WPT;
-  static_assert(G == ROW_GROUPS, "a dequantize unit is 8 groups");
-  const int64_t sg0 = unit * SGS;
+  constexpr int NI = WPT / PARTS;   // groups of a super-group that this unit writes
+  constexpr int G = SGS * NI;
+  static_assert(PARTS >= 1 && WPT % PARTS == 0 && (PARTS == 1 || SGS == 1), "parts divide one super-group");
+  static_assert(G >= 1 && G <= ROW_GROUPS && (G & (G - 1)) == 0, "a dequantize unit is 1, 2, 4 or 8 groups");
+  const int64_t sg0 = unit / PARTS * SGS;
+  const int part = (int)(unit % PARTS);
   const int64_t n_sg = (N + WPT - 1) / WPT;
-  const int64_t g0 = sg0 * WPT;
+  const int64_t g0 = sg0 * WPT + part * NI;   // first group of the unit
   const int rl = l & 15;  // lane within its 16-lane row
   uint32_t w[SGS][W / 4];
 #pragma unroll
@@ -804,6 +808,10 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
       if (live) t = stream_load(reinterpret_cast<const u32x2*>(p));
       w[it][0] = t.x;
       w[it][W / 4 - 1] = t.y;
+    }
+    if (PARTS > 1) {   // this part's fields down to where part 0 has them (the shift is less than a byte)
+#pragma unroll
+      for (int k = 0; k < W / 4; k++) w[it][k] >>= part * NI * BITS;
     }
   }
 
@@ -828,10 +836,10 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
 #pragma unroll
     for (int it = 0; it < SGS; it++) {
 #pragma unroll
-      for (int ni = 0; ni < WPT; ni++) {
-        const int64_t n = (sg0 + it) * WPT + ni;
+      for (int ni = 0; ni < NI; ni++) {
+        const int64_t n = g0 + it * WPT + ni;
         if (n < N) {
-          const int g = it * WPT + ni;
+          const int g = it * NI + ni;
           const uint32_t base4 = (unitbase + (uint32_t)((g * ENT) % LPU)) << 2;
           T v[W];
 #pragma unroll
@@ -879,9 +887,9 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
     }
   }
   // one correctly rounded reciprocal per group and row instead of one per group and lane: row lane j takes
-  // group j & 7 and the row shares the results; when any scale of the wave is outside the range the
+  // group j % G and the row shares the results; when any scale of the wave is outside the range the
   // reciprocal form is valid for, the wave takes the plain division instead
-  const int64_t gm = g0 + (rl & 7);
+  const int64_t gm = g0 + (rl & (G - 1));
   const float s_mine = gm < N ? (float)scale[gm] : 1.0f;
   const float r_mine = 1.0f / s_mine;
   const bool by_reciprocal = __builtin_amdgcn_ballot_w64(!reciprocal_safe(s_mine)) == 0;
@@ -989,8 +997,6 @@ __device__ __forceinline__ void minimax_row(const T* __restrict__ x, int64_t N, 
 // ------------------------------------------------------------------------------------------------
 // Single-tensor kernels.
 // ------------------------------------------------------------------------------------------------
-// groups a single-tensor dequantize unit (a wave for float, half a wave for half) covers
-__host__ __device__ constexpr int dq_supergroups(int bits) { return ROW_GROUPS / (8 / bits); }
 
 // Workgroups go to the 8 XCDs round-robin (workgroup b runs on XCD b % 8) and every XCD streams through its
 // own L2.  With the plain mapping an XCD sees every 8th tile, i.e. addresses in which three bits never
@@ -1050,6 +1056,26 @@ __host__ __device__ constexpr QGeom q_geom(int bits) {
   return Elem<T>::kDtype == GACT_F32 ? f32[k] : Elem<T>::kDtype == GACT_F16 ? f16[k] : b16[k];
 }
 
+// Geometry of the single-tensor dequantize launch for 1, 2, 4 and 8 bit: super-groups per unit, parts a
+// super-group is split into (sgs = 1 then), threads per workgroup, XCD-aware run of tiles.  Units of 8 groups
+// unless 4 measured faster (float 1 bit 31.6 -> 31.1 us at 43 M elements, float 8 bit 29.1 -> 28.9 us at 34 M,
+// half 2 bit 51.7 -> 50.5 us at 134 M, half 8 bit 9.44 -> 9.32 us at 17 M); units of 1 or 2 groups cost 10-150 %:
+// every unit pays its code loads, its table and its divisions.
+struct DqGeom { int sgs, parts, threads, run; };
+#ifndef GACT_DQGEOM_F32
+#define GACT_DQGEOM_F32 {{1, 2, 256, GACT_XCD_RUN_DQ}, {2, 1, 256, GACT_XCD_RUN_DQ}, {4, 1, 256, GACT_XCD_RUN_DQ}, {4, 1, 256, GACT_XCD_RUN_DQ}}
+#endif
+#ifndef GACT_DQGEOM_F16
+#define GACT_DQGEOM_F16 {{1, 1, 256, GACT_XCD_RUN_DQ}, {1, 1, 256, GACT_XCD_RUN_DQ}, {4, 1, 256, GACT_XCD_RUN_DQ}, {4, 1, 256, GACT_XCD_RUN_DQ}}
+#endif
+template <typename T>
+__host__ __device__ constexpr DqGeom dq_geom(int bits) {
+  constexpr DqGeom f32[4] = GACT_DQGEOM_F32, f16[4] = GACT_DQGEOM_F16;
+  const int k = bits == 1 ? 0 : bits == 2 ? 1 : bits == 4 ? 2 : 3;
+  return sizeof(T) == 4 ? f32[k] : f16[k];
+}
+__host__ __device__ constexpr int dq_unit_groups(DqGeom d, int bits) { return d.sgs * (8 / bits) / d.parts; }
+
 template <typename T, int BITS, int NOISE, bool GIVEN>
 __global__ void __launch_bounds__(256)
 quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
@@ -1069,11 +1095,11 @@ __global__ void __launch_bounds__(256)
 dequantize_kernel(const uint8_t* __restrict__ packed, const typename Elem<T>::Stat* __restrict__ scale,
                   const T* __restrict__ mn,
                   int64_t numel, int64_t N, T* __restrict__ out) {
-  constexpr int LPU = GROUP / Elem<T>::kDqWidth;  // lanes per unit of 8 groups: 64 (float) or 32 (half)
-  const int64_t unit = ((int64_t)xcd_tile<GACT_XCD_RUN_DQ>(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x) / LPU;
-  constexpr int SGS = dq_supergroups(BITS);
-  if (unit * ROW_GROUPS >= N) return;
-  dequantize_unit<T, BITS, SGS>(packed, scale, mn, numel, N, unit, threadIdx.x % LPU, out);
+  constexpr DqGeom D = dq_geom<T>(BITS);
+  constexpr int LPU = GROUP / Elem<T>::kDqWidth;  // lanes per unit: 64 (float) or 32 (half)
+  const int64_t unit = ((int64_t)xcd_tile<(uint32_t)D.run>(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x) / LPU;
+  if (unit * dq_unit_groups(D, BITS) >= N) return;
+  dequantize_unit<T, BITS, D.sgs, D.parts>(packed, scale, mn, numel, N, unit, threadIdx.x % LPU, out);
 }
 
 template <typename T>
@@ -1852,11 +1878,12 @@ template <typename T>
 int dispatch_dequantize(int bits, const uint8_t* packed, const typename Elem<T>::Stat* scale, const T* mn,
                         int64_t numel, int64_t N, T* out,
                         hipStream_t stream) {
-  // a unit of 8 groups takes 256 / (16 / sizeof(T)) lanes
-  const int64_t units_per_block = 256 / (GROUP / (16 / (int64_t)sizeof(T)));
-  const int64_t unit_groups = ROW_GROUPS;
+  // a unit takes 256 / (16 / sizeof(T)) lanes
+  const DqGeom d = dq_geom<T>(bits);
+  const int64_t units_per_block = d.threads / (GROUP / (16 / (int64_t)sizeof(T)));
+  const int64_t unit_groups = dq_unit_groups(d, bits);
   const unsigned lds = dequantize_lds_cap(sizeof(T), bits, N);
-  const dim3 grid((unsigned)(((N + unit_groups - 1) / unit_groups + units_per_block - 1) / units_per_block)), block(256);
+  const dim3 grid((unsigned)(((N + unit_groups - 1) / unit_groups + units_per_block - 1) / units_per_block)), block((unsigned)d.threads);
   switch (bits) {
     case 1: hipLaunchKernelGGL((dequantize_kernel<T, 1>), grid, block, lds, stream, packed, scale, mn, numel, N, out); break;
     case 2: hipLaunchKernelGGL((dequantize_kernel<T, 2>), grid, block, lds, stream, packed, scale, mn, numel, N, out); break;
