@@ -186,8 +186,9 @@ def run_workload(torch, name, timer, seed=42, keep_input=False):
 
 def run_ceilings(torch, timer):
     """What this GPU's memory system gives plain streams over config2's tensor (411 MB), in the same run: the
-    runtime's device-to-device copy, a fill, and a pure read (the library's row min/max, which reads the tensor
-    with the fused kernel's access pattern and writes 2 values per 256)."""
+    runtime's device-to-device copy, a fill, a pure read (the library's row min/max, which reads the tensor
+    with the fused kernel's access pattern and writes 2 values per 256), and torch's element-wise conversion
+    kernel at the 8:1 and 1:8 read:write mixes of quantize and dequantize."""
     from gact.cpp_extension import _abi
 
     lib = _abi.lib()
@@ -209,8 +210,20 @@ def run_ceilings(torch, timer):
         _abi.check(lib.gact_minimax(x.data_ptr(), _abi.F32, N, 256, mn.data_ptr(), mx.data_ptr(),
                                     torch.cuda.current_stream().cuda_stream))
 
+    # the traffic mix of quantize / dequantize at 4 bit (8 bytes read per byte written, and the reverse) through
+    # torch's own element-wise kernel: the tensor's bytes as int64, narrowed to int8 and widened back
+    wide, narrow = x.view(torch.int64), torch.empty((x.numel() // 2,), dtype=torch.int8, device="cuda")
+
+    def narrow8(k):
+        narrow.copy_(wide.view(-1))
+
+    def widen8(k):
+        y.view(torch.int64).view(-1).copy_(narrow)
+
     out = {"tensor": "config2's (%d bytes)" % nbytes}
-    for name, fn, moved in (("device_copy", copy, 2 * nbytes), ("fill", fill, nbytes), ("read_minimax", read, nbytes + 8 * N)):
+    for name, fn, moved in (("device_copy", copy, 2 * nbytes), ("fill", fill, nbytes), ("read_minimax", read, nbytes + 8 * N),
+                            ("torch_read8_write1", narrow8, nbytes + nbytes // 8),
+                            ("torch_read1_write8", widen8, nbytes + nbytes // 8)):
         ms, _ = timer(fn)
         out[name] = {"us": ms * 1e3, "gbs": moved / (ms * 1e-3) / 1e9, "frac": moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
     # what a launch costs whatever it moves: one group of 256 elements through the same entry point, replayed the same way

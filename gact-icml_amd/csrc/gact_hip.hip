@@ -624,71 +624,77 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
   typename Elem<T>::Store v[GPR];
   typedef typename Elem<T>::Stat Stat;
   Stat lo_t[GPR], hi_t[GPR], s_t[GPR];
-  if (STAGED && SGR == 1 && WPT > 1 && !GIVEN && NOISE != GACT_NOISE_REF && (n0 + WPT) * GROUP <= numel) {
+  if (STAGED && GPR > 1 && !GIVEN && NOISE != GACT_NOISE_REF && (n0 + GPR) * GROUP <= numel) {
     // All groups whole: the loads in one straight line, then group by group as they arrive: reduce, divide (every
-    // lane for itself), encode.  The work on the first groups overlaps the loads of the later ones within the wave,
-    // which pays where few waves share a SIMD (small tensors) and costs the extra divisions elsewhere.
+    // lane for itself), encode; a super-group goes out when its last group is done.  The work on the first groups
+    // overlaps the loads of the later ones within the wave, which pays where few waves share a SIMD (small tensors)
+    // and costs the extra divisions elsewhere.
 #pragma unroll
-    for (int g = 0; g < WPT; g++)
+    for (int g = 0; g < GPR; g++)
 #pragma unroll
       for (int k = 0; k < CH; k++) Elem<T>::load_chunk(x + (n0 + g) * GROUP + chunk_col<T>(k, i), v[g], k);
     uint32_t bytes[CH][W];
 #pragma unroll
-    for (int k = 0; k < CH; k++)
-#pragma unroll
-      for (int e = 0; e < W; e++) bytes[k][e] = 0;
-#pragma unroll
-    for (int g = 0; g < WPT; g++) {
+    for (int g = 0; g < GPR; g++) {
       const int64_t n = n0 + g;
-      {
-        Stat lo = (Stat)0.0f, hi = (Stat)0.0f;
-        Elem<T>::group_minmax(v[g], lo, hi);
-        const Stat sc = Elem<T>::make_scale(lo, hi, QMAX);
-        if (i == 0) {
-          scale_out[n] = sc;
-          mn_io[n] = Elem<T>::elem_of(lo);
-          if (mx_io) mx_io[n] = Elem<T>::elem_of(hi);
-        }
-        float u[CH][W];
-        if (NOISE == GACT_NOISE_FAST) {
-          fast_noise<T>(n, i, k0, k1, u);
-        } else {
+      const int ni = g % WPT;
+      if (ni == 0) {
 #pragma unroll
-          for (int k = 0; k < CH; k++) {
-            if (NOISE == GACT_NOISE_INJECT) {
-              Elem<T>::load_noise(noise + n * GROUP + chunk_col<T>(k, i), u[k]);
-            } else {
+        for (int k = 0; k < CH; k++)
 #pragma unroll
-              for (int e = 0; e < W; e++) u[k][e] = 0.5f;
-            }
-          }
-        }
+          for (int e = 0; e < W; e++) bytes[k][e] = 0;
+      }
+      Stat lo = (Stat)0.0f, hi = (Stat)0.0f;
+      Elem<T>::group_minmax(v[g], lo, hi);
+      const Stat sc = Elem<T>::make_scale(lo, hi, QMAX);
+      if (i == 0) {
+        scale_out[n] = sc;
+        mn_io[n] = Elem<T>::elem_of(lo);
+        if (mx_io) mx_io[n] = Elem<T>::elem_of(hi);
+      }
+      float u[CH][W];
+      if (NOISE == GACT_NOISE_FAST) {
+        fast_noise<T>(n, i, k0, k1, u);
+      } else {
 #pragma unroll
         for (int k = 0; k < CH; k++) {
-          uint32_t c[W];
-          Elem<T>::template codes<NOISE == GACT_NOISE_CONST, GIVEN>(v[g], k, lo, sc, u[k], c);
+          if (NOISE == GACT_NOISE_INJECT) {
+            Elem<T>::load_noise(noise + n * GROUP + chunk_col<T>(k, i), u[k]);
+          } else {
 #pragma unroll
-          for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (g * BITS);
-        }
-        if (Elem<T>::kRepairsInfiniteScale && __builtin_amdgcn_ballot_w64(Elem<T>::scale_is_inf(sc)) != 0) {
-          if (Elem<T>::scale_is_inf(sc)) {
-#pragma unroll
-            for (int k = 0; k < CH; k++)
-#pragma unroll
-              for (int e = 0; e < W; e++)
-                if (Elem<T>::above(v[g], k, e, lo)) bytes[k][e] |= 0xffffffffu << (g * BITS);
+            for (int e = 0; e < W; e++) u[k][e] = 0.5f;
           }
         }
       }
-      // the codes of this group exist before the next group's loads are waited for
 #pragma unroll
-      for (int k = 0; k < CH; k++)
+      for (int k = 0; k < CH; k++) {
+        uint32_t c[W];
+        Elem<T>::template codes<NOISE == GACT_NOISE_CONST, GIVEN>(v[g], k, lo, sc, u[k], c);
 #pragma unroll
-        for (int e = 0; e < W; e++) asm volatile("" : "+v"(bytes[k][e]));
+        for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (ni * BITS);
+      }
+      if (Elem<T>::kRepairsInfiniteScale && __builtin_amdgcn_ballot_w64(Elem<T>::scale_is_inf(sc)) != 0) {
+        if (Elem<T>::scale_is_inf(sc)) {
+#pragma unroll
+          for (int k = 0; k < CH; k++)
+#pragma unroll
+            for (int e = 0; e < W; e++)
+              if (Elem<T>::above(v[g], k, e, lo)) bytes[k][e] |= 0xffffffffu << (ni * BITS);
+        }
+      }
+      if (ni == WPT - 1) {
+#pragma unroll
+        for (int k = 0; k < CH; k++)
+          Elem<T>::store_codes(packed + (sg0 + g / WPT) * GROUP + chunk_col<T>(k, i), bytes[k]);
+      } else {
+        // the codes of this group exist before the next group's loads are waited for
+#pragma unroll
+        for (int k = 0; k < CH; k++)
+#pragma unroll
+          for (int e = 0; e < W; e++) asm volatile("" : "+v"(bytes[k][e]));
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int k = 0; k < CH; k++) Elem<T>::store_codes(packed + sg0 * GROUP + chunk_col<T>(k, i), bytes[k]);
     return;
   }
 #pragma unroll
