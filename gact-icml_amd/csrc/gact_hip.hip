@@ -603,12 +603,12 @@ __device__ __forceinline__ void fast_noise(int64_t n, int i, uint32_t k0, uint32
 // ------------------------------------------------------------------------------------------------
 // Quantize SGR consecutive super-groups (one 16-lane row): all their groups are loaded first, reduced, and share
 // one scale division per lane; the codes then go out super-group by super-group.
-//   STAGED (one super-group of several whole groups): group by group instead, see below.
+//   STAGE > 0 (rows of whole groups): STAGE groups at a time instead, see below.
 //   GIVEN = false: min/max are reduced here (fused minimax + scale + pack, one read of x).
 //   GIVEN = true : min/max are read from mn_io / mx_io (the pack entry point's contract).
 // Codes follow quantization_cuda_kernel.cu:38-71; see Elem<T>::code1 for the arithmetic.
 // ------------------------------------------------------------------------------------------------
-template <typename T, int BITS, int NOISE, bool GIVEN, int SGR = 1, bool STAGED = false>
+template <typename T, int BITS, int NOISE, bool GIVEN, int SGR = 1, int STAGE = 0>
 __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int64_t numel, int64_t N, int64_t sg0,
                                                     int i, uint8_t* __restrict__ packed,
                                                     typename Elem<T>::Stat* __restrict__ scale_out,
@@ -624,70 +624,97 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
   typename Elem<T>::Store v[GPR];
   typedef typename Elem<T>::Stat Stat;
   Stat lo_t[GPR], hi_t[GPR], s_t[GPR];
-  if (STAGED && GPR > 1 && !GIVEN && NOISE != GACT_NOISE_REF && (n0 + GPR) * GROUP <= numel) {
-    // All groups whole: the loads in one straight line, then group by group as they arrive: reduce, divide (every
-    // lane for itself), encode; a super-group goes out when its last group is done.  The work on the first groups
-    // overlaps the loads of the later ones within the wave, which pays where few waves share a SIMD (small tensors)
-    // and costs the extra divisions elsewhere.
+  if (STAGE > 0 && STAGE < GPR && !GIVEN && NOISE != GACT_NOISE_REF && (n0 + GPR) * GROUP <= numel) {
+    // All groups whole: the loads in one straight line, then STAGE groups at a time as they arrive: reduce, divide
+    // (lane j for group j % STAGE of the stage), encode; a super-group goes out when its last group is done.  The
+    // work on the first groups overlaps the loads of the later ones within the wave, which pays where few waves
+    // share a SIMD (small tensors) and costs the extra divisions elsewhere.
+    static_assert(STAGE <= 0 || (GPR % (STAGE > 0 ? STAGE : 1) == 0 && (STAGE & (STAGE - 1)) == 0), "stages divide the row");
+    constexpr int ST = STAGE > 0 ? STAGE : 1;
 #pragma unroll
     for (int g = 0; g < GPR; g++)
 #pragma unroll
       for (int k = 0; k < CH; k++) Elem<T>::load_chunk(x + (n0 + g) * GROUP + chunk_col<T>(k, i), v[g], k);
     uint32_t bytes[CH][W];
 #pragma unroll
-    for (int g = 0; g < GPR; g++) {
-      const int64_t n = n0 + g;
-      const int ni = g % WPT;
-      if (ni == 0) {
+    for (int g0 = 0; g0 < GPR; g0 += ST) {
+      Stat lo_s[ST], hi_s[ST], sc_s[ST];
 #pragma unroll
-        for (int k = 0; k < CH; k++)
-#pragma unroll
-          for (int e = 0; e < W; e++) bytes[k][e] = 0;
+      for (int j = 0; j < ST; j++) {
+        lo_s[j] = hi_s[j] = (Stat)0.0f;
+        Elem<T>::group_minmax(v[g0 + j], lo_s[j], hi_s[j]);
       }
-      Stat lo = (Stat)0.0f, hi = (Stat)0.0f;
-      Elem<T>::group_minmax(v[g], lo, hi);
-      const Stat sc = Elem<T>::make_scale(lo, hi, QMAX);
-      if (i == 0) {
-        scale_out[n] = sc;
-        mn_io[n] = Elem<T>::elem_of(lo);
-        if (mx_io) mx_io[n] = Elem<T>::elem_of(hi);
-      }
-      float u[CH][W];
-      if (NOISE == GACT_NOISE_FAST) {
-        fast_noise<T>(n, i, k0, k1, u);
-      } else {
+      {
+        const int mine = i & (ST - 1);
+        Stat lo_m = lo_s[0], hi_m = hi_s[0];
 #pragma unroll
-        for (int k = 0; k < CH; k++) {
-          if (NOISE == GACT_NOISE_INJECT) {
-            Elem<T>::load_noise(noise + n * GROUP + chunk_col<T>(k, i), u[k]);
-          } else {
-#pragma unroll
-            for (int e = 0; e < W; e++) u[k][e] = 0.5f;
-          }
+        for (int j = 1; j < ST; j++) {
+          lo_m = (mine == j) ? lo_s[j] : lo_m;
+          hi_m = (mine == j) ? hi_s[j] : hi_m;
+        }
+        const Stat s_m = Elem<T>::make_scale(lo_m, hi_m, QMAX);
+        if (i < ST) {
+          scale_out[n0 + g0 + i] = s_m;
+          mn_io[n0 + g0 + i] = Elem<T>::elem_of(lo_m);
+          if (mx_io) mx_io[n0 + g0 + i] = Elem<T>::elem_of(hi_m);
+        }
+        if (ST == 1) {
+          sc_s[0] = s_m;
+        } else {
+          sc_s[0] = row_bcast<0>(s_m);
+          sc_s[1 % ST] = row_bcast<1>(s_m);
+          if (ST > 2) { sc_s[2 % ST] = row_bcast<2>(s_m); sc_s[3 % ST] = row_bcast<3>(s_m); }
         }
       }
 #pragma unroll
-      for (int k = 0; k < CH; k++) {
-        uint32_t c[W];
-        Elem<T>::template codes<NOISE == GACT_NOISE_CONST, GIVEN>(v[g], k, lo, sc, u[k], c);
-#pragma unroll
-        for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (ni * BITS);
-      }
-      if (Elem<T>::kRepairsInfiniteScale && __builtin_amdgcn_ballot_w64(Elem<T>::scale_is_inf(sc)) != 0) {
-        if (Elem<T>::scale_is_inf(sc)) {
+      for (int j = 0; j < ST; j++) {
+        const int g = g0 + j;
+        const int64_t n = n0 + g;
+        const int ni = g % WPT;
+        if (ni == 0) {
 #pragma unroll
           for (int k = 0; k < CH; k++)
 #pragma unroll
-            for (int e = 0; e < W; e++)
-              if (Elem<T>::above(v[g], k, e, lo)) bytes[k][e] |= 0xffffffffu << (ni * BITS);
+            for (int e = 0; e < W; e++) bytes[k][e] = 0;
+        }
+        float u[CH][W];
+        if (NOISE == GACT_NOISE_FAST) {
+          fast_noise<T>(n, i, k0, k1, u);
+        } else {
+#pragma unroll
+          for (int k = 0; k < CH; k++) {
+            if (NOISE == GACT_NOISE_INJECT) {
+              Elem<T>::load_noise(noise + n * GROUP + chunk_col<T>(k, i), u[k]);
+            } else {
+#pragma unroll
+              for (int e = 0; e < W; e++) u[k][e] = 0.5f;
+            }
+          }
+        }
+#pragma unroll
+        for (int k = 0; k < CH; k++) {
+          uint32_t c[W];
+          Elem<T>::template codes<NOISE == GACT_NOISE_CONST, GIVEN>(v[g], k, lo_s[j], sc_s[j], u[k], c);
+#pragma unroll
+          for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (ni * BITS);
+        }
+        if (Elem<T>::kRepairsInfiniteScale && __builtin_amdgcn_ballot_w64(Elem<T>::scale_is_inf(sc_s[j])) != 0) {
+          if (Elem<T>::scale_is_inf(sc_s[j])) {
+#pragma unroll
+            for (int k = 0; k < CH; k++)
+#pragma unroll
+              for (int e = 0; e < W; e++)
+                if (Elem<T>::above(v[g], k, e, lo_s[j])) bytes[k][e] |= 0xffffffffu << (ni * BITS);
+          }
+        }
+        if (ni == WPT - 1) {
+#pragma unroll
+          for (int k = 0; k < CH; k++)
+            Elem<T>::store_codes(packed + (sg0 + g / WPT) * GROUP + chunk_col<T>(k, i), bytes[k]);
         }
       }
-      if (ni == WPT - 1) {
-#pragma unroll
-        for (int k = 0; k < CH; k++)
-          Elem<T>::store_codes(packed + (sg0 + g / WPT) * GROUP + chunk_col<T>(k, i), bytes[k]);
-      } else {
-        // the codes of this group exist before the next group's loads are waited for
+      if ((g0 + ST) % WPT != 0) {
+        // the codes of this stage exist before the next stage's loads are waited for
 #pragma unroll
         for (int k = 0; k < CH; k++)
 #pragma unroll
@@ -1112,19 +1139,23 @@ struct SeedArg {
 
 // Geometry of the single-tensor quantize launch for an element type and width (1, 2, 4, 8 bit): super-groups per
 // row (a row always issues the loads of all its groups first), threads per workgroup, the XCD-aware run of tiles,
-// and whether a row of whole groups is worked through group by group.  Overridable at compile time
+// and how many groups at a time a row of whole groups is worked through (0: all at once) - `stage` in general,
+// `stage_small` for tensors of fewer than `small_below` groups.  Overridable at compile time
 // (-DGACT_QGEOM_F32=..., _F16, _BF16) for experiments.
-struct QGeom { int sgr, threads, run; bool staged; };
+struct QGeom { int sgr, threads, run, stage, stage_small, small_below; };
 #ifndef GACT_QGEOM_F16
-#define GACT_QGEOM_F16 {{1, 64, 0, false}, {1, 64, 128, false}, {1, 256, 128, false}, {1, 256, 128, false}}
+#define GACT_QGEOM_F16 {{1, 64, 0, 0, 0, 0}, {1, 64, 128, 0, 0, 0}, {1, 256, 128, 0, 0, 0}, {1, 256, 128, 0, 0, 0}}
 #endif
 #ifndef GACT_QGEOM_BF16
-#define GACT_QGEOM_BF16 {{1, 64, 0, false}, {1, 64, 128, false}, {1, 256, 128, false}, {1, 256, 128, false}}
+#define GACT_QGEOM_BF16 {{1, 64, 0, 0, 0, 0}, {1, 64, 128, 0, 0, 0}, {1, 256, 128, 0, 0, 0}, {1, 256, 128, 0, 0, 0}}
 #endif
-// float at 2 and 4 bit works group by group: 4 M elements 5.70 -> 5.51 us (2 bit), 5.88 -> 5.73 us (4 bit), 103 M
-// elements 69.0 -> 67.8 us (2 bit) and unchanged at 4 bit; float at 1 bit (8 divisions per lane) and half lose 3-8 %
+// Staging pays where few waves share a SIMD and costs its extra divisions elsewhere.  float, quantize alone:
+//   1 bit, 4 groups at a time: 8 M elements 9.8 -> 8.4 us, 17 M 14.5 -> 13.6, 34 M unchanged, 43 M 32.0 -> 32.4;
+//   2 bit, group by group: 4 M 5.70 -> 5.51 us, 103 M 69.0 -> 67.8; two at a time is 2 % better still at 4 M and
+//     1-2 % worse from 17 M on;  4 bit, group by group: 4 M 5.88 -> 5.73 us, unchanged at 103 M.
+// half loses 3-8 % group by group at 2 bit and gains or loses 1-2 % otherwise: it keeps the plain order.
 #ifndef GACT_QGEOM_F32
-#define GACT_QGEOM_F32 {{1, 64, 0, false}, {1, 64, 128, true}, {1, 64, 128, true}, {1, 256, 128, false}}
+#define GACT_QGEOM_F32 {{1, 64, 0, 0, 4, 1 << 17}, {1, 64, 128, 1, 2, 1 << 15}, {1, 64, 128, 1, 1, 0}, {1, 256, 128, 0, 0, 0}}
 #endif
 template <typename T>
 __host__ __device__ constexpr QGeom q_geom(int bits) {
@@ -1153,17 +1184,18 @@ __host__ __device__ constexpr DqGeom dq_geom(int bits) {
 }
 __host__ __device__ constexpr int dq_unit_groups(DqGeom d, int bits) { return d.sgs * (8 / bits) / d.parts; }
 
-template <typename T, int BITS, int NOISE, bool GIVEN>
+template <typename T, int BITS, int NOISE, bool GIVEN, bool SMALL = false>
 __global__ void __launch_bounds__(256)
 quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
                 typename Elem<T>::Stat* __restrict__ scale_out, T* mn_io, T* mx_io, SeedArg seed_arg,
                 const float* __restrict__ noise) {
   constexpr QGeom G = q_geom<T>(BITS);
+  constexpr int STAGE = SMALL ? G.stage_small : G.stage;
   constexpr int SGR = NOISE == GACT_NOISE_REF ? 1 : G.sgr;   // the reference stream's code is too long to lay out several times
   const int64_t sg0 = ((int64_t)xcd_tile<(uint32_t)G.run>(blockIdx.x, gridDim.x) * (blockDim.x >> 4) + (threadIdx.x >> 4)) * SGR;
   if (sg0 * (8 / BITS) >= N) return;
   const uint64_t seed = seed_arg.value();
-  quantize_supergroup<T, BITS, NOISE, GIVEN, SGR, G.staged>(x, numel, N, sg0, threadIdx.x & 15, packed, scale_out, mn_io, mx_io,
+  quantize_supergroup<T, BITS, NOISE, GIVEN, SGR, STAGE>(x, numel, N, sg0, threadIdx.x & 15, packed, scale_out, mn_io, mx_io,
                                                   (uint32_t)seed, (uint32_t)(seed >> 32), noise);
 }
 
@@ -1905,6 +1937,24 @@ inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
   return bits == 4 ? 10000u : 0u;
 }
 
+// the kernel of a noise mode; its small-tensor form where the geometry has one (staging is for fused min/max and
+// not for the reference stream)
+template <typename T, int BITS, int NOISE, bool GIVEN>
+void launch_quantize_kernel(bool small, dim3 grid, dim3 block, unsigned lds, hipStream_t stream, const T* x, int64_t numel,
+                            int64_t N, uint8_t* packed, typename Elem<T>::Stat* scale, T* mn, T* mx, SeedArg seed,
+                            const float* noise) {
+  constexpr QGeom G = q_geom<T>(BITS);
+  if constexpr (!GIVEN && NOISE != GACT_NOISE_REF && G.stage_small != G.stage) {
+    if (small) {
+      hipLaunchKernelGGL((quantize_kernel<T, BITS, NOISE, GIVEN, true>), grid, block, lds, stream, x, numel, N, packed,
+                         scale, mn, mx, seed, noise);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((quantize_kernel<T, BITS, NOISE, GIVEN, false>), grid, block, lds, stream, x, numel, N, packed, scale,
+                     mn, mx, seed, noise);
+}
+
 template <typename T, int BITS, bool GIVEN>
 int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, typename Elem<T>::Stat* scale, T* mn, T* mx,
                     int noise_mode,
@@ -1915,22 +1965,19 @@ int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, typen
   row_grid((supergroups(N, BITS) + sgr - 1) / sgr, &grid, &block, G.threads);
   // the reference stream's one Philox block per byte makes the kernel instruction-bound: it wants every wave
   const unsigned lds = noise_mode == GACT_NOISE_REF ? 0u : quantize_lds_cap(sizeof(T), BITS, N);
+  const bool small = N < G.small_below;
   switch (noise_mode) {
     case GACT_NOISE_CONST:
-      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_CONST, GIVEN>), grid, block, lds, stream, x, numel, N,
-                         packed, scale, mn, mx, seed, noise);
+      launch_quantize_kernel<T, BITS, GACT_NOISE_CONST, GIVEN>(small, grid, block, lds, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
       break;
     case GACT_NOISE_INJECT:
-      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_INJECT, GIVEN>), grid, block, lds, stream, x, numel, N,
-                         packed, scale, mn, mx, seed, noise);
+      launch_quantize_kernel<T, BITS, GACT_NOISE_INJECT, GIVEN>(small, grid, block, lds, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
       break;
     case GACT_NOISE_REF:
-      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_REF, GIVEN>), grid, block, lds, stream, x, numel, N,
-                         packed, scale, mn, mx, seed, noise);
+      launch_quantize_kernel<T, BITS, GACT_NOISE_REF, GIVEN>(small, grid, block, lds, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
       break;
     case GACT_NOISE_FAST:
-      hipLaunchKernelGGL((quantize_kernel<T, BITS, GACT_NOISE_FAST, GIVEN>), grid, block, lds, stream, x, numel, N,
-                         packed, scale, mn, mx, seed, noise);
+      launch_quantize_kernel<T, BITS, GACT_NOISE_FAST, GIVEN>(small, grid, block, lds, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
       break;
     default:
       return GACT_EINVAL;
