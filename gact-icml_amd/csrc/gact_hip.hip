@@ -1144,16 +1144,17 @@ struct SeedArg {
 // (-DGACT_QGEOM_F32=..., _F16, _BF16) for experiments.
 struct QGeom { int sgr, threads, run, stage, stage_small, small_below; };
 #ifndef GACT_QGEOM_F16
-#define GACT_QGEOM_F16 {{1, 64, 0, 0, 0, 0}, {1, 64, 128, 0, 0, 0}, {1, 256, 128, 0, 0, 0}, {1, 256, 128, 0, 0, 0}}
+#define GACT_QGEOM_F16 {{1, 64, 0, 4, 4, 0}, {1, 64, 128, 0, 2, 1 << 17}, {1, 256, 128, 0, 0, 0}, {1, 256, 128, 0, 0, 0}}
 #endif
 #ifndef GACT_QGEOM_BF16
-#define GACT_QGEOM_BF16 {{1, 64, 0, 0, 0, 0}, {1, 64, 128, 0, 0, 0}, {1, 256, 128, 0, 0, 0}, {1, 256, 128, 0, 0, 0}}
+#define GACT_QGEOM_BF16 {{1, 64, 0, 4, 4, 0}, {1, 64, 128, 0, 2, 1 << 17}, {1, 256, 128, 0, 0, 0}, {1, 256, 128, 0, 0, 0}}
 #endif
 // Staging pays where few waves share a SIMD and costs its extra divisions elsewhere.  float, quantize alone:
 //   1 bit, 4 groups at a time: 8 M elements 9.8 -> 8.4 us, 17 M 14.5 -> 13.6, 34 M unchanged, 43 M 32.0 -> 32.4;
 //   2 bit, group by group: 4 M 5.70 -> 5.51 us, 103 M 69.0 -> 67.8; two at a time is 2 % better still at 4 M and
 //     1-2 % worse from 17 M on;  4 bit, group by group: 4 M 5.88 -> 5.73 us, unchanged at 103 M.
-// half loses 3-8 % group by group at 2 bit and gains or loses 1-2 % otherwise: it keeps the plain order.
+// half: 1 bit, 4 groups at a time: 4 M elements 6.7 -> 6.3 us, 17 M 11.8 -> 10.5, 67 M 29.0 -> 28.3;  2 bit, two at a
+//   time: 2 % faster up to 17 M, 2 % slower at 67 M and 134 M (group by group: 3-8 % slower);  4 bit: within 1 %.
 #ifndef GACT_QGEOM_F32
 #define GACT_QGEOM_F32 {{1, 64, 0, 0, 4, 1 << 17}, {1, 64, 128, 1, 2, 1 << 15}, {1, 64, 128, 1, 1, 0}, {1, 256, 128, 0, 0, 0}}
 #endif
