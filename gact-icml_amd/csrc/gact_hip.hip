@@ -1030,6 +1030,9 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
 // not depend on the widths.  Quantize: each of the workgroup's 16 rows takes 8 consecutive groups - BITS
 // super-groups - in one go: no loop, 16 KB (half) in flight per wave at every width, one scale division per
 // lane and 8 groups.
+#ifndef GACT_QB_STAGE
+#define GACT_QB_STAGE 0 /* groups at a time in the batched quantize rows (0: all 8 at once) */
+#endif
 template <typename T, int BITS, int NOISE>
 __device__ __forceinline__ void quantize_block128(const T* __restrict__ x, int64_t numel, int64_t N, int64_t lb,
                                                   uint8_t* __restrict__ packed,
@@ -1046,8 +1049,8 @@ __device__ __forceinline__ void quantize_block128(const T* __restrict__ x, int64
         quantize_supergroup<T, BITS, NOISE, false, 1>(x, numel, N, sg0 + q, i, packed, scale_out, mn_out, (T*)nullptr,
                                                       (uint32_t)seed, (uint32_t)(seed >> 32), nullptr);
   } else if (sg0 * WPT < N) {
-    quantize_supergroup<T, BITS, NOISE, false, BITS>(x, numel, N, sg0, i, packed, scale_out, mn_out, (T*)nullptr,
-                                                     (uint32_t)seed, (uint32_t)(seed >> 32), nullptr);
+    quantize_supergroup<T, BITS, NOISE, false, BITS, GACT_QB_STAGE>(x, numel, N, sg0, i, packed, scale_out, mn_out, (T*)nullptr,
+                                                                    (uint32_t)seed, (uint32_t)(seed >> 32), nullptr);
   }
 }
 // Dequantize: two workgroups share a block of 128 groups, 8 units of 8 groups each, so that a unit slot
