@@ -1147,10 +1147,10 @@ struct SeedArg {
 // (-DGACT_QGEOM_F32=..., _F16, _BF16) for experiments.
 struct QGeom { int sgr, threads, run, stage, stage_small, small_below; };
 #ifndef GACT_QGEOM_F16
-#define GACT_QGEOM_F16 {{1, 64, 0, 4, 4, 0}, {1, 64, 128, 0, 2, 1 << 17}, {1, 256, 128, 0, 0, 0}, {1, 256, 128, 0, 0, 0}}
+#define GACT_QGEOM_F16 {{1, 64, 0, 4, 4, 0}, {1, 64, 128, 0, 2, 1 << 17}, {1, 256, 128, 0, 0, 0}, {1, 64, 128, 0, 0, 0}}
 #endif
 #ifndef GACT_QGEOM_BF16
-#define GACT_QGEOM_BF16 {{1, 64, 0, 4, 4, 0}, {1, 64, 128, 0, 2, 1 << 17}, {1, 256, 128, 0, 0, 0}, {1, 256, 128, 0, 0, 0}}
+#define GACT_QGEOM_BF16 {{1, 64, 0, 4, 4, 0}, {1, 64, 128, 0, 2, 1 << 17}, {1, 256, 128, 0, 0, 0}, {1, 64, 128, 0, 0, 0}}
 #endif
 // Staging pays where few waves share a SIMD and costs its extra divisions elsewhere.  float, quantize alone:
 //   1 bit, 4 groups at a time: 8 M elements 9.8 -> 8.4 us, 17 M 14.5 -> 13.6, 34 M unchanged, 43 M 32.0 -> 32.4;
@@ -1158,6 +1158,7 @@ struct QGeom { int sgr, threads, run, stage, stage_small, small_below; };
 //     1-2 % worse from 17 M on;  4 bit, group by group: 4 M 5.88 -> 5.73 us, unchanged at 103 M.
 // half: 1 bit, 4 groups at a time: 4 M elements 6.7 -> 6.3 us, 17 M 11.8 -> 10.5, 67 M 29.0 -> 28.3;  2 bit, two at a
 //   time: 2 % faster up to 17 M, 2 % slower at 67 M and 134 M (group by group: 3-8 % slower);  4 bit: within 1 %.
+//   8 bit in one-wave workgroups: 4 M elements 4.78 -> 4.41 us, 17 M 10.7 -> 10.5, 67 M 32.3 -> 31.8 (4 bit and float 8 bit lose 1-5 % that way).
 #ifndef GACT_QGEOM_F32
 #define GACT_QGEOM_F32 {{1, 64, 0, 0, 4, 1 << 17}, {1, 64, 128, 1, 2, 1 << 15}, {1, 64, 128, 1, 1, 0}, {1, 256, 128, 0, 0, 0}}
 #endif
@@ -2010,7 +2011,8 @@ int dispatch_dequantize(int bits, const uint8_t* packed, const typename Elem<T>:
   const DqGeom d = dq_geom<T>(bits);
   const int64_t units_per_block = d.threads / (GROUP / (16 / (int64_t)sizeof(T)));
   const int64_t unit_groups = dq_unit_groups(d, bits);
-  const unsigned lds = dequantize_lds_cap(sizeof(T), bits, N);
+  // the caps are stated for workgroups of 256 threads
+  const unsigned lds = dequantize_lds_cap(sizeof(T), bits, N) * (unsigned)d.threads / 256u;
   const dim3 grid((unsigned)(((N + unit_groups - 1) / unit_groups + units_per_block - 1) / units_per_block)), block((unsigned)d.threads);
   switch (bits) {
     case 1: hipLaunchKernelGGL((dequantize_kernel<T, 1>), grid, block, lds, stream, packed, scale, mn, numel, N, out); break;
