@@ -1170,16 +1170,20 @@ __host__ __device__ constexpr QGeom q_geom(int bits) {
 }
 
 // Geometry of the single-tensor dequantize launch for 1, 2, 4 and 8 bit: super-groups per unit, parts a
-// super-group is split into (sgs = 1 then), threads per workgroup, XCD-aware run of tiles.  Units of 8 groups
-// unless 4 measured faster (float 1 bit 31.6 -> 31.1 us at 43 M elements, float 8 bit 29.1 -> 28.9 us at 34 M,
-// half 2 bit 51.7 -> 50.5 us at 134 M, half 8 bit 9.44 -> 9.32 us at 17 M); units of 1 or 2 groups cost 10-150 %:
-// every unit pays its code loads, its table and its divisions.
-struct DqGeom { int sgs, parts, threads, run; };
+// super-group is split into (sgs = 1 then), threads per workgroup, XCD-aware run of tiles - and the same pair
+// (sgs, parts) for large tensors (GACT_CAP_FROM_GROUPS groups and more), with the bytes of dynamic LDS a workgroup
+// of 256 threads asks for there without touching them (0: none; see dq_large below).
+// Below that size units are 8 groups unless 4 measured faster (float 1 bit 31.6 -> 31.1 us at 43 M elements, float
+// 8 bit 29.1 -> 28.9 us at 34 M, half 8 bit 9.44 -> 9.32 us at 17 M); units of 1 or 2 groups cost 10-150 %: every
+// unit pays its code loads, its table and its divisions.
+struct DqGeom { int sgs, parts, threads, run, sgs_large, parts_large; unsigned lds_large; };
 #ifndef GACT_DQGEOM_F32
-#define GACT_DQGEOM_F32 {{1, 2, 256, GACT_XCD_RUN_DQ}, {2, 1, 256, GACT_XCD_RUN_DQ}, {4, 1, 256, GACT_XCD_RUN_DQ}, {4, 1, 256, GACT_XCD_RUN_DQ}}
+#define GACT_DQGEOM_F32 {{1, 2, 256, GACT_XCD_RUN_DQ, 1, 1, 53000u}, {2, 1, 256, GACT_XCD_RUN_DQ, 2, 1, 53000u}, \
+                         {4, 1, 256, GACT_XCD_RUN_DQ, 4, 1, 53000u}, {4, 1, 256, GACT_XCD_RUN_DQ, 8, 1, 53000u}}
 #endif
 #ifndef GACT_DQGEOM_F16
-#define GACT_DQGEOM_F16 {{1, 1, 256, GACT_XCD_RUN_DQ}, {1, 1, 256, GACT_XCD_RUN_DQ}, {4, 1, 256, GACT_XCD_RUN_DQ}, {4, 1, 256, GACT_XCD_RUN_DQ}}
+#define GACT_DQGEOM_F16 {{1, 1, 256, GACT_XCD_RUN_DQ, 1, 1, 0u}, {1, 1, 256, GACT_XCD_RUN_DQ, 1, 1, 0u}, \
+                         {4, 1, 256, GACT_XCD_RUN_DQ, 4, 1, 0u}, {4, 1, 256, GACT_XCD_RUN_DQ, 8, 1, 40000u}}
 #endif
 template <typename T>
 __host__ __device__ constexpr DqGeom dq_geom(int bits) {
@@ -1187,7 +1191,9 @@ __host__ __device__ constexpr DqGeom dq_geom(int bits) {
   const int k = bits == 1 ? 0 : bits == 2 ? 1 : bits == 4 ? 2 : 3;
   return sizeof(T) == 4 ? f32[k] : f16[k];
 }
-__host__ __device__ constexpr int dq_unit_groups(DqGeom d, int bits) { return d.sgs * (8 / bits) / d.parts; }
+__host__ __device__ constexpr int dq_unit_groups(DqGeom d, int bits, bool large) {
+  return (large ? d.sgs_large : d.sgs) * (8 / bits) / (large ? d.parts_large : d.parts);
+}
 
 template <typename T, int BITS, int NOISE, bool GIVEN, bool SMALL = false>
 __global__ void __launch_bounds__(256)
@@ -1204,7 +1210,7 @@ quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __re
                                                   (uint32_t)seed, (uint32_t)(seed >> 32), noise);
 }
 
-template <typename T, int BITS>
+template <typename T, int BITS, bool LARGE = false>
 __global__ void __launch_bounds__(256)
 dequantize_kernel(const uint8_t* __restrict__ packed, const typename Elem<T>::Stat* __restrict__ scale,
                   const T* __restrict__ mn,
@@ -1212,8 +1218,9 @@ dequantize_kernel(const uint8_t* __restrict__ packed, const typename Elem<T>::St
   constexpr DqGeom D = dq_geom<T>(BITS);
   constexpr int LPU = GROUP / Elem<T>::kDqWidth;  // lanes per unit: 64 (float) or 32 (half)
   const int64_t unit = ((int64_t)xcd_tile<(uint32_t)D.run>(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x) / LPU;
-  if (unit * dq_unit_groups(D, BITS) >= N) return;
-  dequantize_unit<T, BITS, D.sgs, D.parts>(packed, scale, mn, numel, N, unit, threadIdx.x % LPU, out);
+  if (unit * dq_unit_groups(D, BITS, LARGE) >= N) return;
+  dequantize_unit<T, BITS, LARGE ? D.sgs_large : D.sgs, LARGE ? D.parts_large : D.parts>(packed, scale, mn, numel, N, unit,
+                                                                                       threadIdx.x % LPU, out);
 }
 
 template <typename T>
@@ -1914,29 +1921,23 @@ inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8
 // the other direction into their main direction, and past a point more requests in flight make that mix more
 // expensive for the memory system, not cheaper (a stand-alone kernel that writes 8 KB and reads 1 KB per
 // wave: 88 us for 411 MB at full occupancy, 70 us at 2 waves per SIMD).  The cap is a request for dynamic
-// LDS that the kernels never touch - a CU has 160 KB of it, so 53 000 bytes admit 3 workgroups.
-// Interleaved A/B in both orders on a 411 MB float tensor (us, full occupancy -> capped): dequantize with
-// 3 workgroups of 4 waves per CU 1 bit 77.3 -> 64.5, 2 bit 76.3 -> 69.0, 4 bit 80.0 -> 77.8, 8 bit 83.2 -> 79.3;
-// half 8 bit with 4 workgroups 65.8 -> 62.7; quantize float 4 bit with 16 one-wave workgroups 76.1 -> 71.1.
+// LDS that the kernels never touch - a CU has 160 KB of it, so 53 000 bytes admit 3 workgroups.  What counts is
+// the bytes in flight per CU: the cap goes with units of 8 groups (8 KB of stores per float wave); with units of 4
+// it starves the CU (float 1 bit, 103 M elements: 66 us with units of 8 and the cap, 71 with units of 4 and no cap,
+// 98 with units of 4 and the cap; float 8 bit: 80, 82, 96; half 8 bit, 256 M elements, 4 workgroups per CU: 119, 129,
+// 147).  Hence the geometry table's own entries for large tensors.
+// Interleaved A/B in both orders on a 411 MB float tensor (us, full occupancy -> capped), units of 8 groups:
+// dequantize with 3 workgroups of 4 waves per CU 1 bit 76.3 -> 66.1, 2 bit 76.4 -> 69.6, 4 bit 77.6 -> 74.5,
+// 8 bit 81.7 -> 79.9; quantize float 4 bit with 16 one-wave workgroups 76.1 -> 71.1.
 // The other kernels (all half quantize, float quantize at 1, 2 and 8 bit) and small tensors gain nothing or
 // lose, and keep full occupancy.
-// From 50 M elements on: with buffers that are cold in every cache the cap costs 3-12 % at 8-17 M elements,
-// is neutral at 34 M and gains 2-7 % at 50 M, 3-13 % at 84 M.
+// From 2^17 groups (34 M elements) on: with buffers that are cold in every cache the cap costs 3-12 % at 8-17 M
+// elements, is neutral at 31-34 M and gains 1-7 % from 43 M, 3-13 % at 84 M.
 #ifndef GACT_CAP_FROM_GROUPS
-#define GACT_CAP_FROM_GROUPS (3 << 16)
+#define GACT_CAP_FROM_GROUPS (1 << 17)
 #endif
 constexpr int64_t kCapFromGroups = GACT_CAP_FROM_GROUPS;
-inline unsigned dequantize_lds_cap(size_t elem_size, int bits, int64_t N) {
-  if (N < kCapFromGroups) return 0u;
-#ifndef GACT_DQ_LDS_F32
-#define GACT_DQ_LDS_F32 53000u
-#endif
-#ifndef GACT_DQ_LDS_F16_LOW
-#define GACT_DQ_LDS_F16_LOW 0u
-#endif
-  if (elem_size == 4) return GACT_DQ_LDS_F32;
-  return bits == 8 ? 40000u : GACT_DQ_LDS_F16_LOW;
-}
+inline bool dq_large(int64_t N) { return N >= kCapFromGroups; }
 inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
   if (elem_size != 4 || N < kCapFromGroups) return 0u;
   return bits == 4 ? 10000u : 0u;
@@ -2009,18 +2010,25 @@ int dispatch_dequantize(int bits, const uint8_t* packed, const typename Elem<T>:
                         hipStream_t stream) {
   // a unit takes 256 / (16 / sizeof(T)) lanes
   const DqGeom d = dq_geom<T>(bits);
+  const bool large = dq_large(N);
   const int64_t units_per_block = d.threads / (GROUP / (16 / (int64_t)sizeof(T)));
-  const int64_t unit_groups = dq_unit_groups(d, bits);
+  const int64_t unit_groups = dq_unit_groups(d, bits, large);
   // the caps are stated for workgroups of 256 threads
-  const unsigned lds = dequantize_lds_cap(sizeof(T), bits, N) * (unsigned)d.threads / 256u;
+  const unsigned lds = large ? d.lds_large * (unsigned)d.threads / 256u : 0u;
   const dim3 grid((unsigned)(((N + unit_groups - 1) / unit_groups + units_per_block - 1) / units_per_block)), block((unsigned)d.threads);
+#define GACT_LAUNCH_DQ(B)                                                                                              \
+  if (large)                                                                                                           \
+    hipLaunchKernelGGL((dequantize_kernel<T, B, true>), grid, block, lds, stream, packed, scale, mn, numel, N, out);  \
+  else                                                                                                                 \
+    hipLaunchKernelGGL((dequantize_kernel<T, B, false>), grid, block, lds, stream, packed, scale, mn, numel, N, out)
   switch (bits) {
-    case 1: hipLaunchKernelGGL((dequantize_kernel<T, 1>), grid, block, lds, stream, packed, scale, mn, numel, N, out); break;
-    case 2: hipLaunchKernelGGL((dequantize_kernel<T, 2>), grid, block, lds, stream, packed, scale, mn, numel, N, out); break;
-    case 4: hipLaunchKernelGGL((dequantize_kernel<T, 4>), grid, block, lds, stream, packed, scale, mn, numel, N, out); break;
-    case 8: hipLaunchKernelGGL((dequantize_kernel<T, 8>), grid, block, lds, stream, packed, scale, mn, numel, N, out); break;
+    case 1: GACT_LAUNCH_DQ(1); break;
+    case 2: GACT_LAUNCH_DQ(2); break;
+    case 4: GACT_LAUNCH_DQ(4); break;
+    case 8: GACT_LAUNCH_DQ(8); break;
     default: return GACT_EINVAL;
   }
+#undef GACT_LAUNCH_DQ
   return launch_status();
 }
 

@@ -132,11 +132,13 @@ def test_config3_bert_large_fp16(name, shape, kind, bits):
     cross_check_kernel_paths(x, q, bits, "fast", 7)
 
 
-@pytest.mark.parametrize("dtype,bits", [(torch.float16, 8), (torch.float32, 1), (torch.float32, 8)])
-def test_launches_with_capped_occupancy(dtype, bits):
-    """From 196 608 groups on some kernels are launched with fewer resident waves per CU (a request for dynamic
-    LDS that they never touch): the widths and types whose capped launch no BASELINE workload reaches."""
-    x = gen((196608 + 3, 256), dtype, "relu", 5)
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_large_tensor_launches(dtype, bits):
+    """From 131 072 groups on dequantize takes its large-tensor geometry (units of 8 groups) and some kernels are
+    launched with fewer resident waves per CU (a request for dynamic LDS that they never touch): every type and
+    width just past that size, with a partial last super-group."""
+    x = gen((131072 + 3, 256), dtype, "relu", 5)
     q, out = check_against_oracle(x, bits, "fast", 13)
     check_properties(x, q, out, bits, stochastic=True)
 
