@@ -184,51 +184,54 @@ def run_workload(torch, name, timer, seed=42, keep_input=False):
     return res, (x if keep_input else None)
 
 
-def run_ceilings(torch, timer):
-    """What this GPU's memory system gives plain streams over config2's tensor (411 MB), in the same run: the
-    runtime's device-to-device copy, a fill, a pure read (the library's row min/max, which reads the tensor
-    with the fused kernel's access pattern and writes 2 values per 256), and torch's element-wise conversion
-    kernel at the 8:1 and 1:8 read:write mixes of quantize and dequantize."""
+def run_ceilings(torch, timer, name="config2"):
+    """What this GPU's memory system gives plain streams over a workload's tensor (config2's 411 MB; config1's
+    16 MB, in as many buffer sets as its own measurement rotates over), in the same run: the runtime's
+    device-to-device copy, a fill, a pure read (the library's row min/max, which reads the tensor with the fused
+    kernel's access pattern and writes 2 values per 256), and torch's element-wise conversion kernel at the 8:1
+    and 1:8 read:write mixes of quantize and dequantize."""
     from gact.cpp_extension import _abi
 
     lib = _abi.lib()
-    shape, dtype, _, _, kind, _ = WORKLOADS["config2"]
-    x = make_input(torch, shape, dtype, kind)
-    y = torch.empty_like(x)
-    nbytes = x.numel() * x.element_size()
-    N = x.numel() // 256
-    mn = torch.empty((N,), dtype=x.dtype, device="cuda")
-    mx = torch.empty((N,), dtype=x.dtype, device="cuda")
+    shape, dtype, _, _, kind, _ = WORKLOADS[name]
+    x0 = make_input(torch, shape, dtype, kind)
+    nbytes = x0.numel() * x0.element_size()
+    N = x0.numel() // 256
+    sets = max(1, -(-ROTATE_BYTES // (2 * nbytes + nbytes // 8)))
+    xs = [x0 if r == 0 else x0.clone() for r in range(sets)]
+    ys = [torch.empty_like(x0) for _ in range(sets)]
+    mn = torch.empty((N,), dtype=x0.dtype, device="cuda")
+    mx = torch.empty((N,), dtype=x0.dtype, device="cuda")
 
     def copy(k):
-        y.copy_(x)
+        ys[k % sets].copy_(xs[k % sets])
 
     def fill(k):
-        y.fill_(1.0)
+        ys[k % sets].fill_(1.0)
 
     def read(k):
-        _abi.check(lib.gact_minimax(x.data_ptr(), _abi.F32, N, 256, mn.data_ptr(), mx.data_ptr(),
+        _abi.check(lib.gact_minimax(xs[k % sets].data_ptr(), _abi.F32, N, 256, mn.data_ptr(), mx.data_ptr(),
                                     torch.cuda.current_stream().cuda_stream))
 
     # the traffic mix of quantize / dequantize at 4 bit (8 bytes read per byte written, and the reverse) through
     # torch's own element-wise kernel: the tensor's bytes as int64, narrowed to int8 and widened back
-    wide, narrow = x.view(torch.int64), torch.empty((x.numel() // 2,), dtype=torch.int8, device="cuda")
+    narrow = [torch.empty((x0.numel() // 2,), dtype=torch.int8, device="cuda") for _ in range(sets)]
 
     def narrow8(k):
-        narrow.copy_(wide.view(-1))
+        narrow[k % sets].copy_(xs[k % sets].view(torch.int64).view(-1))
 
     def widen8(k):
-        y.view(torch.int64).view(-1).copy_(narrow)
+        ys[k % sets].view(torch.int64).view(-1).copy_(narrow[k % sets])
 
-    out = {"tensor": "config2's (%d bytes)" % nbytes}
-    for name, fn, moved in (("device_copy", copy, 2 * nbytes), ("fill", fill, nbytes), ("read_minimax", read, nbytes + 8 * N),
-                            ("torch_read8_write1", narrow8, nbytes + nbytes // 8),
-                            ("torch_read1_write8", widen8, nbytes + nbytes // 8)):
+    out = {"tensor": "%s's (%d bytes)" % (name, nbytes), "buffer_sets": sets}
+    for key, fn, moved in (("device_copy", copy, 2 * nbytes), ("fill", fill, nbytes), ("read_minimax", read, nbytes + 8 * N),
+                           ("torch_read8_write1", narrow8, nbytes + nbytes // 8),
+                           ("torch_read1_write8", widen8, nbytes + nbytes // 8)):
         ms, _ = timer(fn)
-        out[name] = {"us": ms * 1e3, "gbs": moved / (ms * 1e-3) / 1e9, "frac": moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        out[key] = {"us": ms * 1e3, "gbs": moved / (ms * 1e-3) / 1e9, "frac": moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
     # what a launch costs whatever it moves: one group of 256 elements through the same entry point, replayed the same way
-    tiny, tq = x.reshape(-1)[:256], torch.empty((65,), dtype=torch.int8, device="cuda")
-    ts, tm = torch.empty((1,), dtype=x.dtype, device="cuda"), torch.empty((1,), dtype=x.dtype, device="cuda")
+    tiny, tq = x0.reshape(-1)[:256], torch.empty((65,), dtype=torch.int8, device="cuda")
+    ts, tm = torch.empty((1,), dtype=x0.dtype, device="cuda"), torch.empty((1,), dtype=x0.dtype, device="cuda")
 
     def one_group(k):
         _abi.check(lib.gact_quantize(tiny.data_ptr(), _abi.F32, 256, 2, _abi.NOISE_CONST, 0, None, tq.data_ptr(),
@@ -441,7 +444,11 @@ def main():
                               "step": {"us": c3_us, "gbs": 2 * c3_bytes / c3_us / 1e3,
                                        "frac": 2 * c3_bytes / c3_us / 1e3 / HBM_PEAK_GBS}}
         line["configs"] = configs
-        line["ceilings"] = run_ceilings(torch, timer)
+        line["ceilings"] = run_ceilings(torch, timer, "config2")
+        torch.cuda.empty_cache()
+        # the same plain streams at the headline workload's size, where the launch and the ramp of a 16 MB
+        # stream count: what a kernel that only reads (or only fills) this tensor takes
+        line["ceilings_headline"] = run_ceilings(torch, timer, "config1")
         torch.cuda.empty_cache()
     if not args.no_cpu and x is not None:
         line["cpu_baseline"] = cpu_baseline(torch, x, res["bits"], res["rng_stream"])
