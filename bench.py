@@ -184,12 +184,12 @@ def run_workload(torch, name, timer, seed=42, keep_input=False):
     return res, (x if keep_input else None)
 
 
-def run_ceilings(torch, timer, name="config2"):
+def run_ceilings(torch, timer, name="config2", full=True):
     """What this GPU's memory system gives plain streams over a workload's tensor (config2's 411 MB; config1's
     16 MB, in as many buffer sets as its own measurement rotates over), in the same run: the runtime's
     device-to-device copy, a fill, a pure read (the library's row min/max, which reads the tensor with the fused
     kernel's access pattern and writes 2 values per 256), and torch's element-wise conversion kernel at the 8:1
-    and 1:8 read:write mixes of quantize and dequantize."""
+    and 1:8 read:write mixes of quantize and dequantize.  full = False: the fill and the pure read only."""
     from gact.cpp_extension import _abi
 
     lib = _abi.lib()
@@ -210,12 +210,12 @@ def run_ceilings(torch, timer, name="config2"):
         ys[k % sets].fill_(1.0)
 
     def read(k):
-        _abi.check(lib.gact_minimax(xs[k % sets].data_ptr(), _abi.F32, N, 256, mn.data_ptr(), mx.data_ptr(),
+        _abi.check(lib.gact_minimax(xs[k % sets].data_ptr(), _abi.dtype_code(x0.dtype), N, 256, mn.data_ptr(), mx.data_ptr(),
                                     torch.cuda.current_stream().cuda_stream))
 
     # the traffic mix of quantize / dequantize at 4 bit (8 bytes read per byte written, and the reverse) through
     # torch's own element-wise kernel: the tensor's bytes as int64, narrowed to int8 and widened back
-    narrow = [torch.empty((x0.numel() // 2,), dtype=torch.int8, device="cuda") for _ in range(sets)]
+    narrow = [torch.empty((nbytes // 8 if full else 8,), dtype=torch.int8, device="cuda") for _ in range(sets)]
 
     def narrow8(k):
         narrow[k % sets].copy_(xs[k % sets].view(torch.int64).view(-1))
@@ -224,9 +224,12 @@ def run_ceilings(torch, timer, name="config2"):
         ys[k % sets].view(torch.int64).view(-1).copy_(narrow[k % sets])
 
     out = {"tensor": "%s's (%d bytes)" % (name, nbytes), "buffer_sets": sets}
-    for key, fn, moved in (("device_copy", copy, 2 * nbytes), ("fill", fill, nbytes), ("read_minimax", read, nbytes + 8 * N),
+    esize = x0.element_size()
+    for key, fn, moved in (("device_copy", copy, 2 * nbytes), ("fill", fill, nbytes), ("read_minimax", read, nbytes + 2 * esize * N),
                            ("torch_read8_write1", narrow8, nbytes + nbytes // 8),
                            ("torch_read1_write8", widen8, nbytes + nbytes // 8)):
+        if not full and key not in ("fill", "read_minimax"):
+            continue
         ms, _ = timer(fn)
         out[key] = {"us": ms * 1e3, "gbs": moved / (ms * 1e-3) / 1e9, "frac": moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
     # what a launch costs whatever it moves: one group of 256 elements through the same entry point, replayed the same way
@@ -237,8 +240,9 @@ def run_ceilings(torch, timer, name="config2"):
         _abi.check(lib.gact_quantize(tiny.data_ptr(), _abi.F32, 256, 2, _abi.NOISE_CONST, 0, None, tq.data_ptr(),
                                      ts.data_ptr(), tm.data_ptr(), None, torch.cuda.current_stream().cuda_stream))
 
-    ms, _ = timer(one_group)
-    out["launch_floor_us"] = ms * 1e3
+    if full:
+        ms, _ = timer(one_group)
+        out["launch_floor_us"] = ms * 1e3
     return out
 
 
@@ -450,6 +454,11 @@ def main():
         # stream count: what a kernel that only reads (or only fills) this tensor takes
         line["ceilings_headline"] = run_ceilings(torch, timer, "config1")
         torch.cuda.empty_cache()
+        # and the fill and the pure read at the sizes of the other small and mid-sized workloads
+        line["ceilings_by_size"] = {}
+        for name in ("config3-hidden", "config3-gelu", "config4"):
+            line["ceilings_by_size"][name] = run_ceilings(torch, timer, name, full=False)
+            torch.cuda.empty_cache()
     if not args.no_cpu and x is not None:
         line["cpu_baseline"] = cpu_baseline(torch, x, res["bits"], res["rng_stream"])
     else:

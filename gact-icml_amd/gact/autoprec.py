@@ -108,10 +108,11 @@ class AutoPrecision:
             g_c = self._get_grad(backprop)
         finally:
             q.bits[l] = kept
-        sens = max(_sq_dist(g_a, g_b), 2 * max(_sq_dist(g_a, g_c), _sq_dist(g_b, g_c)))
-        if not torch.isfinite(sens) or sens > SENSITIVITY_CAP:
-            return SENSITIVITY_CAP
-        return sens.item()
+        # a 0-d tensor on the gradients' device: comparing or reading it here would wait for the three passes,
+        # the caller reads all tensors' values back at once
+        sens = torch.maximum(_sq_dist(g_a, g_b), 2 * torch.maximum(_sq_dist(g_a, g_c), _sq_dist(g_b, g_c)))
+        cap = torch.full_like(sens, SENSITIVITY_CAP)
+        return torch.where(torch.isfinite(sens) & (sens <= SENSITIVITY_CAP), sens, cap)
 
     def _predicted_variance(self, shift):
         C = np.array([self.C[l] for l in self.C])
@@ -134,8 +135,14 @@ class AutoPrecision:
         adapting = self.iter % self.adapt_interval == 0
         if adapting:
             print('GACT: Initializing AutoPrec..., run extra %d iters' % (len(self.quantizer.bits)))
-            for l in list(self.quantizer.bits):
-                self.C[l] = self._sensitivity_of(l, backprop)
+            # the probes of all tensors are queued without a host synchronisation between them (the reference
+            # reads every sensitivity back as soon as its three passes are queued); one read-back at the end
+            layers = list(self.quantizer.bits)
+            sens = [self._sensitivity_of(l, backprop) for l in layers]
+            if sens:
+                values = torch.stack([v.double() for v in sens]).tolist()
+                for l, v in zip(layers, values):
+                    self.C[l] = SENSITIVITY_CAP if v >= SENSITIVITY_CAP else v
             self.refresh_bits()
 
         if adapting and self.debug:
