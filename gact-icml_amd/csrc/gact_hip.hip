@@ -603,12 +603,12 @@ __device__ __forceinline__ void fast_noise(int64_t n, int i, uint32_t k0, uint32
 // ------------------------------------------------------------------------------------------------
 // Quantize SGR consecutive super-groups (one 16-lane row): all their groups are loaded first, reduced, and share
 // one scale division per lane; the codes then go out super-group by super-group.
-//   STAGE > 0 (rows of whole groups): STAGE groups at a time instead, see below.
+//   STAGE > 0 (rows of whole groups): STAGE groups at a time instead, see below; LAZY: each stage issues its own loads.
 //   GIVEN = false: min/max are reduced here (fused minimax + scale + pack, one read of x).
 //   GIVEN = true : min/max are read from mn_io / mx_io (the pack entry point's contract).
 // Codes follow quantization_cuda_kernel.cu:38-71; see Elem<T>::code1 for the arithmetic.
 // ------------------------------------------------------------------------------------------------
-template <typename T, int BITS, int NOISE, bool GIVEN, int SGR = 1, int STAGE = 0>
+template <typename T, int BITS, int NOISE, bool GIVEN, int SGR = 1, int STAGE = 0, bool LAZY = false>
 __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int64_t numel, int64_t N, int64_t sg0,
                                                     int i, uint8_t* __restrict__ packed,
                                                     typename Elem<T>::Stat* __restrict__ scale_out,
@@ -628,16 +628,26 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
     // All groups whole: the loads in one straight line, then STAGE groups at a time as they arrive: reduce, divide
     // (lane j for group j % STAGE of the stage), encode; a super-group goes out when its last group is done.  The
     // work on the first groups overlaps the loads of the later ones within the wave, which pays where few waves
-    // share a SIMD (small tensors) and costs the extra divisions elsewhere.
+    // share a SIMD (small tensors) and costs the extra divisions elsewhere.  LAZY: a stage's loads are issued when
+    // the stage begins (the compiler still hoists what its register budget allows), which suits the
+    // instruction-heavy half kernels once several waves share a SIMD.
     static_assert(STAGE <= 0 || (GPR % (STAGE > 0 ? STAGE : 1) == 0 && (STAGE & (STAGE - 1)) == 0), "stages divide the row");
     constexpr int ST = STAGE > 0 ? STAGE : 1;
+    if (!LAZY) {
 #pragma unroll
-    for (int g = 0; g < GPR; g++)
+      for (int g = 0; g < GPR; g++)
 #pragma unroll
-      for (int k = 0; k < CH; k++) Elem<T>::load_chunk(x + (n0 + g) * GROUP + chunk_col<T>(k, i), v[g], k);
+        for (int k = 0; k < CH; k++) Elem<T>::load_chunk(x + (n0 + g) * GROUP + chunk_col<T>(k, i), v[g], k);
+    }
     uint32_t bytes[CH][W];
 #pragma unroll
     for (int g0 = 0; g0 < GPR; g0 += ST) {
+      if (LAZY) {
+#pragma unroll
+        for (int j = 0; j < ST; j++)
+#pragma unroll
+          for (int k = 0; k < CH; k++) Elem<T>::load_chunk(x + (n0 + g0 + j) * GROUP + chunk_col<T>(k, i), v[g0 + j], k);
+      }
       Stat lo_s[ST], hi_s[ST], sc_s[ST];
 #pragma unroll
       for (int j = 0; j < ST; j++) {
@@ -1143,14 +1153,15 @@ struct SeedArg {
 // Geometry of the single-tensor quantize launch for an element type and width (1, 2, 4, 8 bit): super-groups per
 // row (a row always issues the loads of all its groups first), threads per workgroup, the XCD-aware run of tiles,
 // and how many groups at a time a row of whole groups is worked through (0: all at once) - `stage` in general,
-// `stage_small` for tensors of fewer than `small_below` groups.  Overridable at compile time
+// `stage_small` for tensors of fewer than `small_below` groups - with each stage issuing its own loads (`lazy`,
+// `lazy_small`) instead of the row issuing all of them first.  Overridable at compile time
 // (-DGACT_QGEOM_F32=..., _F16, _BF16) for experiments.
-struct QGeom { int sgr, threads, run, stage, stage_small, small_below; };
+struct QGeom { int sgr, threads, run, stage, stage_small, small_below; bool lazy, lazy_small; };
 #ifndef GACT_QGEOM_F16
-#define GACT_QGEOM_F16 {{1, 64, 0, 4, 4, 0}, {1, 64, 128, 0, 2, 1 << 17}, {1, 256, 128, 0, 0, 0}, {1, 64, 128, 0, 0, 0}}
+#define GACT_QGEOM_F16 {{1, 64, 0, 4, 4, 1 << 15, true, false}, {1, 64, 128, 0, 2, 1 << 17, false, true}, {1, 256, 128, 0, 0, 0, false, false}, {1, 64, 128, 0, 0, 0, false, false}}
 #endif
 #ifndef GACT_QGEOM_BF16
-#define GACT_QGEOM_BF16 {{1, 64, 0, 4, 4, 0}, {1, 64, 128, 0, 2, 1 << 17}, {1, 256, 128, 0, 0, 0}, {1, 64, 128, 0, 0, 0}}
+#define GACT_QGEOM_BF16 {{1, 64, 0, 4, 4, 1 << 15, true, false}, {1, 64, 128, 0, 2, 1 << 17, false, true}, {1, 256, 128, 0, 0, 0, false, false}, {1, 64, 128, 0, 0, 0, false, false}}
 #endif
 // Staging pays where few waves share a SIMD and costs its extra divisions elsewhere.  float, quantize alone:
 //   1 bit, 4 groups at a time: 8 M elements 9.8 -> 8.4 us, 17 M 14.5 -> 13.6, 34 M unchanged, 43 M 32.0 -> 32.4;
@@ -1159,8 +1170,11 @@ struct QGeom { int sgr, threads, run, stage, stage_small, small_below; };
 // half: 1 bit, 4 groups at a time: 4 M elements 6.7 -> 6.3 us, 17 M 11.8 -> 10.5, 67 M 29.0 -> 28.3;  2 bit, two at a
 //   time: 2 % faster up to 17 M, 2 % slower at 67 M and 134 M (group by group: 3-8 % slower);  4 bit: within 1 %.
 //   8 bit in one-wave workgroups: 4 M elements 4.78 -> 4.41 us, 17 M 10.7 -> 10.5, 67 M 32.3 -> 31.8 (4 bit and float 8 bit lose 1-5 % that way).
+//   stages that issue their own loads: 1 bit 4 M elements 6.27 -> 6.67 us, 17 M 10.4 -> 10.1, 34 M 16.3 -> 15.9, 134 M 49.8 -> 49.0
+//   (hence from 2^15 groups on);  2 bit 4 M unchanged, 17 M 10.0 -> 9.2, 26 M 13.8 -> 12.9.  float: 1 bit 4 M 6.5 -> 7.5 us,
+//   17 M 13.6 -> 12.8, 26 M unchanged; 2 and 4 bit within 2 % either way: not used.
 #ifndef GACT_QGEOM_F32
-#define GACT_QGEOM_F32 {{1, 64, 0, 0, 4, 1 << 17}, {1, 64, 128, 1, 2, 1 << 15}, {1, 64, 128, 1, 1, 0}, {1, 256, 128, 0, 0, 0}}
+#define GACT_QGEOM_F32 {{1, 64, 0, 0, 4, 1 << 17, false, false}, {1, 64, 128, 1, 2, 1 << 15, false, false}, {1, 64, 128, 1, 1, 0, false, false}, {1, 256, 128, 0, 0, 0, false, false}}
 #endif
 template <typename T>
 __host__ __device__ constexpr QGeom q_geom(int bits) {
@@ -1202,11 +1216,12 @@ quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __re
                 const float* __restrict__ noise) {
   constexpr QGeom G = q_geom<T>(BITS);
   constexpr int STAGE = SMALL ? G.stage_small : G.stage;
+  constexpr bool LAZY = SMALL ? G.lazy_small : G.lazy;
   constexpr int SGR = NOISE == GACT_NOISE_REF ? 1 : G.sgr;   // the reference stream's code is too long to lay out several times
   const int64_t sg0 = ((int64_t)xcd_tile<(uint32_t)G.run>(blockIdx.x, gridDim.x) * (blockDim.x >> 4) + (threadIdx.x >> 4)) * SGR;
   if (sg0 * (8 / BITS) >= N) return;
   const uint64_t seed = seed_arg.value();
-  quantize_supergroup<T, BITS, NOISE, GIVEN, SGR, STAGE>(x, numel, N, sg0, threadIdx.x & 15, packed, scale_out, mn_io, mx_io,
+  quantize_supergroup<T, BITS, NOISE, GIVEN, SGR, STAGE, LAZY>(x, numel, N, sg0, threadIdx.x & 15, packed, scale_out, mn_io, mx_io,
                                                   (uint32_t)seed, (uint32_t)(seed >> 32), noise);
 }
 
@@ -1950,7 +1965,7 @@ void launch_quantize_kernel(bool small, dim3 grid, dim3 block, unsigned lds, hip
                             int64_t N, uint8_t* packed, typename Elem<T>::Stat* scale, T* mn, T* mx, SeedArg seed,
                             const float* noise) {
   constexpr QGeom G = q_geom<T>(BITS);
-  if constexpr (!GIVEN && NOISE != GACT_NOISE_REF && G.stage_small != G.stage) {
+  if constexpr (!GIVEN && NOISE != GACT_NOISE_REF && (G.stage_small != G.stage || G.lazy_small != G.lazy)) {
     if (small) {
       hipLaunchKernelGGL((quantize_kernel<T, BITS, NOISE, GIVEN, true>), grid, block, lds, stream, x, numel, N, packed,
                          scale, mn, mx, seed, noise);
