@@ -1185,19 +1185,24 @@ __host__ __device__ constexpr QGeom q_geom(int bits) {
 
 // Geometry of the single-tensor dequantize launch for 1, 2, 4 and 8 bit: super-groups per unit, parts a
 // super-group is split into (sgs = 1 then), threads per workgroup, XCD-aware run of tiles - and the same pair
-// (sgs, parts) for large tensors (GACT_CAP_FROM_GROUPS groups and more), with the bytes of dynamic LDS a workgroup
-// of 256 threads asks for there without touching them (0: none; see dq_large below).
-// Below that size units are 8 groups unless 4 measured faster (float 1 bit 31.6 -> 31.1 us at 43 M elements, float
-// 8 bit 29.1 -> 28.9 us at 34 M, half 8 bit 9.44 -> 9.32 us at 17 M); units of 1 or 2 groups cost 10-150 %: every
-// unit pays its code loads, its table and its divisions.
-struct DqGeom { int sgs, parts, threads, run, sgs_large, parts_large; unsigned lds_large; };
+// (sgs, parts) for large tensors (`large_from` groups and more), with the bytes of dynamic LDS a workgroup
+// of 256 threads asks for there without touching them (0: none; see the occupancy caps below).
+// Units are 4 or 8 groups; units of 1 or 2 groups cost 10-150 %: every unit pays its code loads, its table and its
+// divisions.  Dequantize alone, us, units of 4 against units of 8 (no cap), by groups in the tensor:
+//   float 1 bit  65 536: 13.95 / 12.29   100 000: 20.0 / 18.4    (2 and 4 bit alike: 8)
+//   float 8 bit  65 536: 15.76 / 15.98   100 000: 23.2 / 23.7    (4, and 8 with the cap from 2^17 groups)
+//   half  1 bit  16 384: 3.86 / 4.36   65 536: 7.36 / 7.87   100 000: 11.3 / 11.3   130 000: 14.2 / 13.3
+//   half  2 bit  16 384: 3.87 / 4.73   65 536: 7.41 / 8.15   130 000: 14.5 / 13.8   1 M: 94.6 / 99.4   (4 throughout)
+//   half  4 bit  16 384: 4.39 / 5.05   65 536: 8.08 / 8.95   100 000: 13.1 / 12.5   130 000: 15.8 / 15.2
+//   half  8 bit  65 536: 9.21 / 9.40   130 000: 18.0 / 18.2
+struct DqGeom { int sgs, parts, threads, run, sgs_large, parts_large; unsigned lds_large; int large_from; };
 #ifndef GACT_DQGEOM_F32
-#define GACT_DQGEOM_F32 {{1, 2, 256, GACT_XCD_RUN_DQ, 1, 1, 53000u}, {2, 1, 256, GACT_XCD_RUN_DQ, 2, 1, 53000u}, \
-                         {4, 1, 256, GACT_XCD_RUN_DQ, 4, 1, 53000u}, {4, 1, 256, GACT_XCD_RUN_DQ, 8, 1, 53000u}}
+#define GACT_DQGEOM_F32 {{1, 1, 256, GACT_XCD_RUN_DQ, 1, 1, 53000u, 1 << 17}, {2, 1, 256, GACT_XCD_RUN_DQ, 2, 1, 53000u, 1 << 17}, \
+                         {4, 1, 256, GACT_XCD_RUN_DQ, 4, 1, 53000u, 1 << 17}, {4, 1, 256, GACT_XCD_RUN_DQ, 8, 1, 53000u, 1 << 17}}
 #endif
 #ifndef GACT_DQGEOM_F16
-#define GACT_DQGEOM_F16 {{1, 1, 256, GACT_XCD_RUN_DQ, 1, 1, 0u}, {1, 1, 256, GACT_XCD_RUN_DQ, 1, 1, 0u}, \
-                         {4, 1, 256, GACT_XCD_RUN_DQ, 4, 1, 0u}, {4, 1, 256, GACT_XCD_RUN_DQ, 8, 1, 40000u}}
+#define GACT_DQGEOM_F16 {{1, 2, 256, GACT_XCD_RUN_DQ, 1, 1, 0u, 3 << 15}, {1, 1, 256, GACT_XCD_RUN_DQ, 1, 1, 0u, 1 << 17}, \
+                         {2, 1, 256, GACT_XCD_RUN_DQ, 4, 1, 0u, 3 << 15}, {4, 1, 256, GACT_XCD_RUN_DQ, 8, 1, 40000u, 1 << 17}}
 #endif
 template <typename T>
 __host__ __device__ constexpr DqGeom dq_geom(int bits) {
@@ -1946,15 +1951,14 @@ inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8
 // 8 bit 81.7 -> 79.9; quantize float 4 bit with 16 one-wave workgroups 76.1 -> 71.1.
 // The other kernels (all half quantize, float quantize at 1, 2 and 8 bit) and small tensors gain nothing or
 // lose, and keep full occupancy.
-// From 2^17 groups (34 M elements) on: with buffers that are cold in every cache the cap costs 3-12 % at 8-17 M
-// elements, is neutral at 31-34 M and gains 1-7 % from 43 M, 3-13 % at 84 M.
-#ifndef GACT_CAP_FROM_GROUPS
-#define GACT_CAP_FROM_GROUPS (1 << 17)
+// From 2^17 groups (34 M elements) on (`large_from` in the geometry table): with buffers that are cold in every cache
+// the cap costs 3-12 % at 8-26 M elements, is neutral at 31-34 M and gains 1-7 % from 43 M, 3-13 % at 84 M.
+// Quantize, float 4 bit: capped from 98 304 groups on (100 000 groups: 21.3 -> 20.3 us, 170 000: 34.3 -> 31.9; 65 536: 14.5 -> 14.8).
+#ifndef GACT_QCAP_FROM_GROUPS
+#define GACT_QCAP_FROM_GROUPS (3 << 15)
 #endif
-constexpr int64_t kCapFromGroups = GACT_CAP_FROM_GROUPS;
-inline bool dq_large(int64_t N) { return N >= kCapFromGroups; }
 inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
-  if (elem_size != 4 || N < kCapFromGroups) return 0u;
+  if (elem_size != 4 || N < GACT_QCAP_FROM_GROUPS) return 0u;
   return bits == 4 ? 10000u : 0u;
 }
 
@@ -2025,7 +2029,7 @@ int dispatch_dequantize(int bits, const uint8_t* packed, const typename Elem<T>:
                         hipStream_t stream) {
   // a unit takes 256 / (16 / sizeof(T)) lanes
   const DqGeom d = dq_geom<T>(bits);
-  const bool large = dq_large(N);
+  const bool large = N >= d.large_from;
   const int64_t units_per_block = d.threads / (GROUP / (16 / (int64_t)sizeof(T)));
   const int64_t unit_groups = dq_unit_groups(d, bits, large);
   // the caps are stated for workgroups of 256 threads
