@@ -1158,10 +1158,10 @@ struct SeedArg {
 // (-DGACT_QGEOM_F32=..., _F16, _BF16) for experiments.
 struct QGeom { int sgr, threads, run, stage, stage_small, small_below; bool lazy, lazy_small; };
 #ifndef GACT_QGEOM_F16
-#define GACT_QGEOM_F16 {{1, 64, 0, 4, 4, 1 << 15, true, false}, {1, 64, 128, 0, 2, 1 << 17, false, true}, {1, 256, 128, 0, 0, 0, false, false}, {1, 64, 128, 0, 0, 0, false, false}}
+#define GACT_QGEOM_F16 {{1, 64, 0, 4, 4, 1 << 15, true, false}, {1, 64, 128, 2, 2, 0, true, true}, {1, 256, 128, 1, 1, 0, true, true}, {1, 64, 128, 0, 0, 0, false, false}}
 #endif
 #ifndef GACT_QGEOM_BF16
-#define GACT_QGEOM_BF16 {{1, 64, 0, 4, 4, 1 << 15, true, false}, {1, 64, 128, 0, 2, 1 << 17, false, true}, {1, 256, 128, 0, 0, 0, false, false}, {1, 64, 128, 0, 0, 0, false, false}}
+#define GACT_QGEOM_BF16 {{1, 64, 0, 4, 4, 1 << 15, true, false}, {1, 64, 128, 2, 2, 0, true, true}, {1, 256, 128, 1, 1, 0, true, true}, {1, 64, 128, 0, 0, 0, false, false}}
 #endif
 // Staging pays where few waves share a SIMD and costs its extra divisions elsewhere.  float, quantize alone:
 //   1 bit, 4 groups at a time: 8 M elements 9.8 -> 8.4 us, 17 M 14.5 -> 13.6, 34 M unchanged, 43 M 32.0 -> 32.4;
@@ -1171,10 +1171,12 @@ struct QGeom { int sgr, threads, run, stage, stage_small, small_below; bool lazy
 //   time: 2 % faster up to 17 M, 2 % slower at 67 M and 134 M (group by group: 3-8 % slower);  4 bit: within 1 %.
 //   8 bit in one-wave workgroups: 4 M elements 4.78 -> 4.41 us, 17 M 10.7 -> 10.5, 67 M 32.3 -> 31.8 (4 bit and float 8 bit lose 1-5 % that way).
 //   stages that issue their own loads: 1 bit 4 M elements 6.27 -> 6.67 us, 17 M 10.4 -> 10.1, 34 M 16.3 -> 15.9, 134 M 49.8 -> 49.0
-//   (hence from 2^15 groups on);  2 bit 4 M unchanged, 17 M 10.0 -> 9.2, 26 M 13.8 -> 12.9.  float: 1 bit 4 M 6.5 -> 7.5 us,
-//   17 M 13.6 -> 12.8, 26 M unchanged; 2 and 4 bit within 2 % either way: not used.
+//   (hence from 2^15 groups on);  2 bit, two at a time: 4 M unchanged, 17 M 10.0 -> 9.2, 26 M 13.8 -> 12.9, 134 M 51.0 -> 49.5,
+//   256 M 93.0 -> 91.5 (bfloat16 67 M: 27.8 -> 26.4);  4 bit, group by group: 8 M 6.66 -> 6.3, 67 M and 256 M within 1 %.
+//   float: 1 bit, four at a time: 4 M 6.5 -> 7.5 us, 17 M 13.6 -> 12.8, 103 M 69.3 -> 67.5, 256 M 170 -> 167 (from 2^15 groups on);
+//   4 bit group by group: 4 M 5.64 -> 5.41, 8 M 8.29 -> 8.15, larger within 1 %;  2 bit within 2 % either way: not used.
 #ifndef GACT_QGEOM_F32
-#define GACT_QGEOM_F32 {{1, 64, 0, 0, 4, 1 << 17, false, false}, {1, 64, 128, 1, 2, 1 << 15, false, false}, {1, 64, 128, 1, 1, 0, false, false}, {1, 256, 128, 0, 0, 0, false, false}}
+#define GACT_QGEOM_F32 {{1, 64, 0, 4, 4, 1 << 15, true, false}, {1, 64, 128, 1, 2, 1 << 15, false, false}, {1, 64, 128, 1, 1, 0, true, true}, {1, 256, 128, 0, 0, 0, false, false}}
 #endif
 template <typename T>
 __host__ __device__ constexpr QGeom q_geom(int bits) {
