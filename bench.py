@@ -11,8 +11,8 @@ Bytes are the algorithmic input + output bytes: numel*sizeof(T) + packed bytes +
 Timing.  The K steps of a block are recorded once into a HIP graph (the launches go through the C ABI on
 the capturing stream) and the graph is replayed between two events on that stream; blocks are repeated
 until at least one second has been measured (the rule of the reference's tests/timeit_v2.py:246-257), the
-mean over all timed steps is reported.  A tensor whose buffers would fit the 256 MB last-level cache is
-given several buffer sets used in rotation, so that every step streams from and to HBM.  The duration of
+mean over all timed steps is reported.  Every workload is
+given several buffer sets used in rotation (4 GB between two uses of a buffer), so that every step streams from and to HBM.  The duration of
 each kernel comes from the same construction with K launches of that kernel alone; `roofline` is the
 slower of the two kernels of the headline workload.  `cpu_baseline` is the C restatement of the reference
 arithmetic (oracle/) with OpenMP on the host cores.
@@ -44,8 +44,11 @@ TRAFFIC_BYTES = {
 
 BASELINE_METRIC = "quantize+dequantize GB/s and % of HBM peak, 1×MI355X, 2-bit group=256"
 
-# a workload whose buffers are smaller than this is timed over several buffer sets in rotation
-ROTATE_BYTES = 800 * 1000 * 1000
+# A workload is timed over as many buffer sets, used in rotation, as it takes to touch this many bytes before a
+# buffer comes round again.  The GPU's last-level cache holds 256 MB and does not evict in strict LRU order: with
+# 0.8 GB between reuses a 411 MB tensor still read 3-4 % faster (and a 173 MB one was written 8 % faster) than
+# from HBM; the figures stop moving at 3 GB.
+ROTATE_BYTES = 4 * 1000 * 1000 * 1000
 
 WORKLOADS = {
     # name: (shape, dtype, bits, rng_stream, data kind, description)
@@ -87,43 +90,51 @@ def algorithmic_bytes(numel, esize, bits, scale_esize=None):
 
 
 class Timer:
-    """Mean duration of fn(k) over blocks of `steps` calls, at least MIN_SECONDS of them."""
+    """Mean duration of fn(k) over blocks of `steps` calls, at least MIN_SECONDS of them.  `period` is the
+    number of distinct k the workload tells apart (its buffer sets): when it exceeds `steps`, consecutive blocks
+    continue the count, so that all of them come round whatever `steps` is."""
 
     def __init__(self, torch, steps, warmup, min_seconds, graph=True):
         self.torch, self.steps, self.warmup, self.min_seconds, self.graph = torch, steps, warmup, min_seconds, graph
 
-    def __call__(self, fn):
+    def __call__(self, fn, period=1):
         torch = self.torch
         for k in range(self.warmup):
             fn(k)
         torch.cuda.synchronize()
-        block = None
+        n_blocks = max(1, min(64, -(-period // self.steps)))
+        blocks = None
         if self.graph:
-            # the block's launches, recorded once on a side stream (capture cannot run on the null stream)
-            block = torch.cuda.CUDAGraph()
+            # every block's launches, recorded once on a side stream (capture cannot run on the null stream)
+            blocks = []
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
-                with torch.cuda.graph(block, stream=side):
-                    for k in range(self.steps):
-                        fn(k)
+                for b in range(n_blocks):
+                    g = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(g, stream=side):
+                        for k in range(self.steps):
+                            fn(b * self.steps + k)
+                    blocks.append(g)
             torch.cuda.current_stream().wait_stream(side)
-            block.replay()      # untimed: the first replay uploads the graph
+            for g in blocks:    # untimed: the first replay uploads the graph
+                g.replay()
             torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        total_ms, calls = 0.0, 0
+        total_ms, calls, b = 0.0, 0, 0
         t_begin = time.perf_counter()
         while True:
             e0.record()
-            if block is not None:
-                block.replay()
+            if blocks is not None:
+                blocks[b].replay()
             else:
                 for k in range(self.steps):
-                    fn(k)
+                    fn(b * self.steps + k)
             e1.record()
             e1.synchronize()
             total_ms += e0.elapsed_time(e1)
             calls += self.steps
+            b = (b + 1) % n_blocks
             if time.perf_counter() - t_begin >= self.min_seconds:
                 break
         return total_ms / calls, calls
@@ -169,9 +180,9 @@ def run_workload(torch, name, timer, seed=42, keep_input=False, rotate=True):
 
     for k in range(sets):   # every set holds valid codes before a dequantize-only loop reads them
         step(k)
-    step_ms, timed_steps = timer(step)
-    q_ms, _ = timer(quantize)
-    d_ms, _ = timer(dequantize)
+    step_ms, timed_steps = timer(step, sets)
+    q_ms, _ = timer(quantize, sets)
+    d_ms, _ = timer(dequantize, sets)
 
     per_dir = algorithmic_bytes(numel, esize, bits, 4 if x.dtype == torch.bfloat16 else None)
     gbs = lambda ms: per_dir / (ms * 1e-3) / 1e9
@@ -231,7 +242,7 @@ def run_ceilings(torch, timer, name="config2", full=True):
                            ("torch_read1_write8", widen8, nbytes + nbytes // 8)):
         if not full and key not in ("fill", "read_minimax"):
             continue
-        ms, _ = timer(fn)
+        ms, _ = timer(fn, sets)
         out[key] = {"us": ms * 1e3, "gbs": moved / (ms * 1e-3) / 1e9, "frac": moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
     # what a launch costs whatever it moves: one group of 256 elements through the same entry point, replayed the same way
     tiny, tq = x0.reshape(-1)[:256], torch.empty((65,), dtype=torch.int8, device="cuda")
