@@ -130,23 +130,25 @@ __device__ __forceinline__ void stream_store(V v, V* p) {
 #endif
 }
 
-// The dequantized tensor leaves through buffer stores whose cache policy the kernel chooses: nontemporal AND
-// written through at system scope (sc0 sc1 nt).  The plain nontemporal store the compiler emits for
-// __builtin_nontemporal_store lets the L2 collect the lines first, which costs a write stream 6-9 % on float
-// tensors (dequantize, 103 M elements at 4 bit: 74.7 -> 70.4 us; 43 M at 1 bit: 30.3 -> 27.4 us; half: unchanged).
+// The dequantized tensor leaves through buffer stores whose cache policy the kernel chooses: nontemporal, and for
+// every type and width but float at 1 bit also written through at system scope (sc0 sc1 nt).  The plain nontemporal
+// store the compiler emits for __builtin_nontemporal_store lets the L2 collect the lines first, which costs a float
+// write stream up to 6 % (dequantize alone, buffers cold in every cache: 4 bit 103 M elements 75.5 -> 71.3 us, 256 M
+// 183.4 -> 172.4; 8 bit 1 %; 2 bit equal; 17 M elements 1-3 % at every width; half 0-2 %), while float at 1 bit,
+// whose stream has the smallest share of reads, loses 3-4 % by it from 50 M elements on (66.3 -> 68.5 us at 103 M).
 // A window is a buffer resource over the bytes from a wave-uniform base to the end of the tensor (at most 4 GB of
 // them: offsets inside a window are 32 bit), so a store past the end of the tensor is dropped by the hardware.
-#ifndef GACT_DQ_STORE_AUX
-#define GACT_DQ_STORE_AUX 19 /* cache-policy bits of the buffer store: 1 sc0, 2 nt, 16 sc1 */
-#endif
+#define GACT_STORE_NT 2          /* cache-policy bits of a buffer store: 1 sc0, 2 nt, 16 sc1 */
+#define GACT_STORE_NT_SYSTEM 19
 struct OutWindow {
   __amdgpu_buffer_rsrc_t rsrc;
   __device__ __forceinline__ OutWindow(void* base, int64_t bytes) {
     const uint32_t n = bytes <= 0 ? 0u : bytes > 0xffffffffLL ? 0xffffffffu : (uint32_t)bytes;
     rsrc = __builtin_amdgcn_make_buffer_rsrc(base, 0, (int)n, 0x00020000);
   }
+  template <int POLICY>
   __device__ __forceinline__ void store16(u32x4 v, uint32_t byte_offset) const {
-    __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, (int)byte_offset, 0, GACT_DQ_STORE_AUX);
+    __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, (int)byte_offset, 0, POLICY);
   }
 };
 __device__ __forceinline__ int64_t wave_first(int64_t v) {
@@ -296,9 +298,10 @@ template <> struct Elem<float> {
   }
   __device__ static __forceinline__ float from_bits(uint32_t b) { return __builtin_bit_cast(float, b); }
   static constexpr int kDqWidth = 4;  // columns per dequantize lane: one 16-byte store
+  template <int POLICY>
   __device__ static __forceinline__ void store_dq(const OutWindow& w, uint32_t byte_offset, const float (&v)[4]) {
     f32x4 a = {v[0], v[1], v[2], v[3]};
-    w.store16(__builtin_bit_cast(u32x4, a), byte_offset);
+    w.template store16<POLICY>(__builtin_bit_cast(u32x4, a), byte_offset);
   }
 };
 
@@ -448,11 +451,12 @@ template <> struct Elem<f16> {
   }
   __device__ static __forceinline__ f16 from_bits(uint32_t b) { return __builtin_bit_cast(f16, (uint16_t)b); }
   static constexpr int kDqWidth = 8;  // columns per dequantize lane: one 16-byte store
+  template <int POLICY>
   __device__ static __forceinline__ void store_dq(const OutWindow& w, uint32_t byte_offset, const f16 (&v)[8]) {
     f16x8 a;
 #pragma unroll
     for (int e = 0; e < 8; e++) a[e] = v[e];
-    w.store16(__builtin_bit_cast(u32x4, a), byte_offset);
+    w.template store16<POLICY>(__builtin_bit_cast(u32x4, a), byte_offset);
   }
 };
 
@@ -522,12 +526,13 @@ template <> struct Elem<bf16> {
   }
   __device__ static __forceinline__ bf16 from_bits(uint32_t b) { return __builtin_bit_cast(bf16, (uint16_t)b); }
   static constexpr int kDqWidth = 8;
+  template <int POLICY>
   __device__ static __forceinline__ void store_dq(const OutWindow& w, uint32_t byte_offset, const bf16 (&v)[8]) {
     typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
     bf16x8 a;
 #pragma unroll
     for (int e = 0; e < 8; e++) a[e] = v[e];
-    w.store16(__builtin_bit_cast(u32x4, a), byte_offset);
+    w.template store16<POLICY>(__builtin_bit_cast(u32x4, a), byte_offset);
   }
 };
 
@@ -932,6 +937,7 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
   const int64_t n_sg = (N + WPT - 1) / WPT;
   const int64_t g0 = sg0 * WPT + part * NI;   // first group of the unit
   const int rl = l & 15;  // lane within its 16-lane row
+  constexpr int POLICY = (sizeof(T) == 4 && BITS == 1) ? GACT_STORE_NT : GACT_STORE_NT_SYSTEM;
   // the wave's output window starts at the first group of its first unit (a wave holds one or two units, in order)
   const int64_t window_first = wave_first(g0) * GROUP;
   const OutWindow window(out + window_first, (numel - window_first) * (int64_t)sizeof(T));
@@ -988,7 +994,7 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
           }
           const int64_t at = n * GROUP + W * l;
           if (n * GROUP + GROUP <= numel) {
-            Elem<T>::store_dq(window, (uint32_t)((at - window_first) * (int64_t)sizeof(T)), v);
+            Elem<T>::template store_dq<POLICY>(window, (uint32_t)((at - window_first) * (int64_t)sizeof(T)), v);
           } else {
 #pragma unroll
             for (int e = 0; e < W; e++)
@@ -1053,7 +1059,7 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
       }
       const int64_t at = n * GROUP + W * l;
       if (n * GROUP + GROUP <= numel) {
-        Elem<T>::store_dq(window, (uint32_t)((at - window_first) * (int64_t)sizeof(T)), v);
+        Elem<T>::template store_dq<POLICY>(window, (uint32_t)((at - window_first) * (int64_t)sizeof(T)), v);
       } else {
 #pragma unroll
         for (int e = 0; e < W; e++)
@@ -1186,10 +1192,10 @@ struct SeedArg {
 // (-DGACT_QGEOM_F32=..., _F16, _BF16) for experiments.
 struct QGeom { int sgr, threads, run, stage, stage_small, small_below; bool lazy, lazy_small; };
 #ifndef GACT_QGEOM_F16
-#define GACT_QGEOM_F16 {{1, 64, 0, 4, 4, 1 << 15, true, false}, {1, 64, 128, 2, 2, 0, true, true}, {1, 256, 128, 1, 1, 0, true, true}, {1, 64, 128, 0, 0, 0, false, false}}
+#define GACT_QGEOM_F16 {{1, 64, 0, 4, 4, 1 << 15, true, false}, {1, 64, 128, 2, 2, 0, true, true}, {1, 64, 128, 1, 1, 0, true, true}, {1, 64, 128, 0, 0, 0, false, false}}
 #endif
 #ifndef GACT_QGEOM_BF16
-#define GACT_QGEOM_BF16 {{1, 64, 0, 4, 4, 1 << 15, true, false}, {1, 64, 128, 2, 2, 0, true, true}, {1, 256, 128, 1, 1, 0, true, true}, {1, 64, 128, 0, 0, 0, false, false}}
+#define GACT_QGEOM_BF16 {{1, 64, 0, 4, 4, 1 << 15, true, false}, {1, 64, 128, 2, 2, 0, true, true}, {1, 64, 128, 1, 1, 0, true, true}, {1, 64, 128, 0, 0, 0, false, false}}
 #endif
 // Staging pays where few waves share a SIMD and costs its extra divisions elsewhere.  float, quantize alone:
 //   1 bit, 4 groups at a time: 8 M elements 9.8 -> 8.4 us, 17 M 14.5 -> 13.6, 34 M unchanged, 43 M 32.0 -> 32.4;
@@ -1223,7 +1229,7 @@ __host__ __device__ constexpr QGeom q_geom(int bits) {
 //   float 8 bit  65 536: 15.76 / 15.98   100 000: 23.2 / 23.7    (4, and 8 with the cap from 2^17 groups)
 //   half  1 bit  16 384: 3.86 / 4.36   65 536: 7.36 / 7.87   100 000: 11.3 / 11.3   130 000: 14.2 / 13.3
 //   half  2 bit  16 384: 3.87 / 4.73   65 536: 7.41 / 8.15   130 000: 14.5 / 13.8   1 M: 94.6 / 99.4   (4 throughout)
-//   half  4 bit  16 384: 4.39 / 5.05   65 536: 8.08 / 8.95   100 000: 13.1 / 12.5   130 000: 15.8 / 15.2
+//   half  4 bit  16 384: 4.39 / 5.05   65 536: 8.08 / 8.95   200 000: 24.0 / 24.0   401 408: 45.0 / 46.7   1 M: 105.1 / 106.7
 //   half  8 bit  65 536: 9.21 / 9.40   130 000: 18.0 / 18.2
 struct DqGeom { int sgs, parts, threads, run, sgs_large, parts_large; unsigned lds_large; int large_from; };
 #ifndef GACT_DQGEOM_F32
@@ -1232,7 +1238,7 @@ struct DqGeom { int sgs, parts, threads, run, sgs_large, parts_large; unsigned l
 #endif
 #ifndef GACT_DQGEOM_F16
 #define GACT_DQGEOM_F16 {{1, 2, 256, GACT_XCD_RUN_DQ, 1, 1, 0u, 3 << 15}, {1, 1, 256, GACT_XCD_RUN_DQ, 1, 1, 0u, 1 << 17}, \
-                         {2, 1, 256, GACT_XCD_RUN_DQ, 4, 1, 0u, 3 << 15}, {4, 1, 256, GACT_XCD_RUN_DQ, 8, 1, 40000u, 1 << 17}}
+                         {2, 1, 256, GACT_XCD_RUN_DQ, 2, 1, 0u, 3 << 15}, {4, 1, 256, GACT_XCD_RUN_DQ, 8, 1, 40000u, 1 << 17}}
 #endif
 template <typename T>
 __host__ __device__ constexpr DqGeom dq_geom(int bits) {
