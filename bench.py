@@ -36,10 +36,10 @@ MIN_SECONDS = 1.0      # every timed loop runs at least this long
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size
 # in the same runs (profiles/<workload>_*.txt name the runs and the factors); absent = no counter run
 TRAFFIC_BYTES = {
-    ("config1", "quantize"): 18.05e6,    # 16.87 MB read + 1.18 MB written; algorithmic 17.96 MB
-    ("config1", "dequantize"): 18.01e6,  # 1.23 MB read + 16.78 MB written
-    ("config2", "quantize"): 466.95e6,   # 411.1 MB read + 55.8 MB written; algorithmic 465.6 MB
-    ("config2", "dequantize"): 465.75e6, # 54.7 MB read + 411.1 MB written
+    ("config1", "quantize"): 18.05e6,    # 16.85 MB read + 1.20 MB written; algorithmic 17.96 MB
+    ("config1", "dequantize"): 18.02e6,  # 1.25 MB read + 16.78 MB written
+    ("config2", "quantize"): 468.90e6,   # 411.1 MB read + 57.8 MB written; algorithmic 465.6 MB
+    ("config2", "dequantize"): 465.70e6, # 54.7 MB read + 411.0 MB written
 }
 
 BASELINE_METRIC = "quantize+dequantize GB/s and % of HBM peak, 1×MI355X, 2-bit group=256"
