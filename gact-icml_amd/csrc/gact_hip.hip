@@ -2003,13 +2003,21 @@ inline int64_t supergroups(int64_t N, int bits) { return (N + 8 / bits - 1) / (8
 // lose, and keep full occupancy.
 // From 2^17 groups (34 M elements) on (`large_from` in the geometry table): with buffers that are cold in every cache
 // the cap costs 3-12 % at 8-26 M elements, is neutral at 31-34 M and gains 1-7 % from 43 M, 3-13 % at 84 M.
-// Quantize, float 4 bit: capped from 98 304 groups on (100 000 groups: 21.3 -> 20.3 us, 170 000: 34.3 -> 31.9; 65 536: 14.5 -> 14.8).
+// Quantize, float: 4 bit capped at 16 one-wave workgroups per CU from 98 304 groups on (100 000 groups: 21.1 -> 20.9 us,
+// 200 000: 40.1 -> 37.9, 401 408: 77.4 -> 72.6, 1 M: 191.5 -> 177.8; 65 536: 14.6 -> 14.65), 2 bit at 8 from 196 608 groups on
+// (262 144 groups: 47.6 -> 46.2 us, 401 408: 72.2 -> 69.1, 1 M: 177.3 -> 165.3; 131 072: 25.3 -> 26.1).  Buffers cold in
+// every cache.  1 and 8 bit gain 1-2 % at most, half loses at 4 and 8 bit and gains 1-2 % at 1 and 2 bit: left alone.
 #ifndef GACT_QCAP_FROM_GROUPS
 #define GACT_QCAP_FROM_GROUPS (3 << 15)
 #endif
+#ifndef GACT_QCAP2_FROM_GROUPS
+#define GACT_QCAP2_FROM_GROUPS (3 << 16)
+#endif
 inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
-  if (elem_size != 4 || N < GACT_QCAP_FROM_GROUPS) return 0u;
-  return bits == 4 ? 10000u : 0u;
+  if (elem_size != 4) return 0u;
+  if (bits == 4) return N >= GACT_QCAP_FROM_GROUPS ? 10000u : 0u;
+  if (bits == 2) return N >= GACT_QCAP2_FROM_GROUPS ? 20000u : 0u;
+  return 0u;
 }
 
 // the kernel of a noise mode; its small-tensor form where the geometry has one (staging is for fused min/max and
