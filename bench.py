@@ -11,11 +11,17 @@ Bytes are the algorithmic input + output bytes: numel*sizeof(T) + packed bytes +
 Timing.  The K steps of a block are recorded once into a HIP graph (the launches go through the C ABI on
 the capturing stream) and the graph is replayed between two events on that stream; blocks are repeated
 until at least one second has been measured (the rule of the reference's tests/timeit_v2.py:246-257), the
-mean over all timed steps is reported.  Every workload is
-given several buffer sets used in rotation (4 GB between two uses of a buffer), so that every step streams from and to HBM.  The duration of
+mean over all timed steps is reported.  Every workload is given several buffer sets used in rotation (4 GB
+between two uses of a buffer, whatever K is), so that every step streams from and to HBM.  The duration of
 each kernel comes from the same construction with K launches of that kernel alone; `roofline` is the
 slower of the two kernels of the headline workload.  `cpu_baseline` is the C restatement of the reference
 arithmetic (oracle/) with OpenMP on the host cores.
+
+Beside the workloads the line carries what plain streams reach in the same run: `ceilings` (device copy, fill,
+pure read, torch's element-wise kernel at the 8:1 and 1:8 read:write mixes, and the duration of a one-group
+launch, on config2's tensor), `ceilings_headline` (the same on config1's tensor) and `ceilings_by_size` (fill and
+pure read at the sizes of the mid-sized workloads); `configs["config1-cached"]` is the headline tensor with one
+buffer set.
 
 Prints ONE JSON line.
 """
