@@ -11,10 +11,11 @@
 // chunk, or the float chunks of a pair of neighbouring lanes (which swap the halves they need) - and, mirrored,
 // the 8 columns half a group further on, which the same lane owns.
 //
-// Dequantize has no reduction, so a unit of 8 consecutive groups goes to a whole wave (float: lane l owns
+// Dequantize has no reduction, so a unit of 4 or 8 consecutive groups goes to a whole wave (float: lane l owns
 // columns 4l .. 4l+3) or half a wave (half: 8l .. 8l+7): one 16-byte store per lane and group, every store
-// instruction writing whole groups contiguously.  At 1, 2 and 4 bit the 8 * 2^bits possible values of a unit
-// are tabulated once across its lanes and fetched with ds_bpermute.
+// instruction writing whole groups contiguously.  At 1, 2 and 4 bit the possible values of a unit (2^bits per
+// group) are tabulated once across its lanes and fetched with ds_bpermute.  The stores are buffer stores whose
+// cache policy the kernel chooses (nontemporal, written through at system scope).
 //
 // Element types: float and half as in the reference; bfloat16 (an addition) is quantized as the float
 // values it holds, in the half layout.
