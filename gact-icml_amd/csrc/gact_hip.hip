@@ -1118,10 +1118,12 @@ __device__ __forceinline__ void dequantize_block128(const uint8_t* __restrict__ 
 
 // Row min/max only (the minimax entry point at D = 256): a 16-lane row takes MINIMAX_ROW_GROUPS consecutive
 // groups, issues all their loads, reduces them one after the other and lets lane g store the results of group g.
-// 2 groups per row (8 KB per float wave) read fastest: float, buffers cold in every cache, 1 / 2 / 4 / 8 groups per
-// row: 4 M elements 4.62 / 4.76 / 5.43 / 5.94 us, 43 M 26.7 / 26.6 / 28.8 / 31.9, 103 M 60.9 / 61.0 / 61.9 / 65.6;
-// half 17 M 7.60 / 7.11 / 7.27 / 8.39, 134 M 40.4 / 40.0 / 40.3 / 41.3.
-#define MINIMAX_ROW_GROUPS 2
+// One group per row in one-wave workgroups (4 KB per float wave) reads fastest.  float, buffers cold in every cache,
+// 1 group per row in 64-thread workgroups / 2 in 256 / 4 in 256 / 8 in 256: 4 M elements 4.68 / 4.81 / 5.44 / 5.94 us,
+// 43 M 26.6 / 26.9 / 29.0 / 31.9, 103 M 60.3 / 61.6 / 61.8 / 65.6, 256 M 148.9 / 155.1 / 155.6 / 159; half 17 M
+// 6.81 / 7.16 / 7.30 / 8.39, 256 M 72.3 / 74.8 / 75.7 / 77.7.
+#define MINIMAX_ROW_GROUPS 1
+#define MINIMAX_THREADS 64
 template <typename T>
 __device__ __forceinline__ void minimax_row(const T* __restrict__ x, int64_t N, int64_t row, int i,
                                             T* __restrict__ mn, T* __restrict__ mx) {
@@ -2220,7 +2222,7 @@ int gact_minimax(const void* data, int dtype, int64_t N, int64_t D, void* mn, vo
   hipStream_t s = (hipStream_t)stream;
   if (D == GROUP && aligned16(data)) {
     dim3 grid, block;
-    row_grid((N + MINIMAX_ROW_GROUPS - 1) / MINIMAX_ROW_GROUPS, &grid, &block);
+    row_grid((N + MINIMAX_ROW_GROUPS - 1) / MINIMAX_ROW_GROUPS, &grid, &block, MINIMAX_THREADS);
     if (dtype == GACT_F32)
       hipLaunchKernelGGL((minimax256_kernel<float>), grid, block, 0, s, (const float*)data, N, (float*)mn, (float*)mx);
     else
