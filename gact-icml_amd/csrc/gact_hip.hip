@@ -1694,10 +1694,74 @@ __device__ __forceinline__ uint32_t sortable_key(float k) {
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
+// Bitonic sort of M = R * NT candidate slots, descending, by a workgroup of NT threads (M and NT powers of two,
+// NT >= 64).  Thread t keeps slots t, NT + t, ... in registers: partners NT or more apart are its own registers,
+// partners less than a wave apart are reached with a shuffle, and only the passes in between go through LDS and
+// a barrier (512 slots by 512 threads: 6 of 45 passes).
+template <int R, int JR>
+__device__ __forceinline__ void prec_exchange_own(uint64_t (&v)[R], int tid, int NT, int k) {
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    if ((r & JR) == 0 && (r | JR) < R) {
+      const bool descending = ((r * NT + tid) & k) == 0;
+      const uint64_t a = v[r], b = v[r | JR];
+      const uint64_t larger = a > b ? a : b, smaller = a > b ? b : a;
+      v[r] = descending ? larger : smaller;   // slot r is the lower one of the pair
+      v[r | JR] = descending ? smaller : larger;
+    }
+  }
+}
+template <int R>
+__device__ __forceinline__ void prec_sort_slots(uint64_t* cand, int tid, int NT, int M) {
+  uint64_t v[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) v[r] = cand[r * NT + tid];
+  for (int k = 2; k <= M; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      if (j >= NT) {
+        switch (j / NT) {
+          case 1: prec_exchange_own<R, 1>(v, tid, NT, k); break;
+          case 2: prec_exchange_own<R, 2>(v, tid, NT, k); break;
+          case 4: prec_exchange_own<R, 4>(v, tid, NT, k); break;
+          default: prec_exchange_own<R, 8>(v, tid, NT, k); break;
+        }
+        continue;
+      }
+      uint64_t o[R];
+      if (j >= 64) {
+#pragma unroll
+        for (int r = 0; r < R; r++) cand[r * NT + tid] = v[r];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < R; r++) o[r] = cand[(r * NT + tid) ^ j];
+        __syncthreads();
+      } else {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          const uint32_t lo32 = (uint32_t)__shfl_xor((int)(uint32_t)v[r], j, 64);
+          const uint32_t hi32 = (uint32_t)__shfl_xor((int)(uint32_t)(v[r] >> 32), j, 64);
+          o[r] = ((uint64_t)hi32 << 32) | lo32;
+        }
+      }
+      // the lower slot of a pair keeps the larger key where the run descends, the smaller where it ascends
+      const bool lower = (tid & j) == 0;
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        const bool descending = ((r * NT + tid) & k) == 0;
+        const uint64_t larger = v[r] > o[r] ? v[r] : o[r], smaller = v[r] > o[r] ? o[r] : v[r];
+        v[r] = (descending == lower) ? larger : smaller;
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; r++) cand[r * NT + tid] = v[r];
+  __syncthreads();
+}
+
 // The greedy pops candidates (tensor i, step s) in descending (key, i) order.  A tensor's steps have
 // strictly decreasing keys, so that order is the descending sort of ALL candidate steps by
 // (key, index, earlier step first); the loop `while (b_sum > target) pop` then takes a prefix of it.
-// One workgroup of 256 or 1024 threads: build up to 4 candidates per tensor, bitonic-sort them in LDS,
+// One workgroup, one thread per candidate slot up to 1024: build up to 4 candidates per tensor, bitonic-sort them,
 // prefix-sum the savings (integers, exact in double), apply the prefix.  Falls back to the sequential
 // loop when that order argument does not hold.
 __global__ void __launch_bounds__(PREC_THREADS)
@@ -1767,18 +1831,12 @@ calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, cons
     if (tid < 64) calc_precision_sequential(b_s, reinterpret_cast<float*>(cand), C, w, L, b_sum0, target, &rc);
   } else {
     // bitonic sort, descending
-    for (int k = 2; k <= M; k <<= 1) {
-      for (int j = k >> 1; j > 0; j >>= 1) {
-        for (int t = tid; t < M; t += NT) {
-          const int o = t ^ j;
-          if (o > t) {
-            const uint64_t x = cand[t], y = cand[o];
-            const bool descending = (t & k) == 0;
-            if (descending ? x < y : x > y) { cand[t] = y; cand[o] = x; }
-          }
-        }
-        __syncthreads();
-      }
+    switch (M / NT) {
+      case 1: prec_sort_slots<1>(cand, tid, NT, M); break;
+      case 2: prec_sort_slots<2>(cand, tid, NT, M); break;
+      case 4: prec_sort_slots<4>(cand, tid, NT, M); break;
+      case 8: prec_sort_slots<8>(cand, tid, NT, M); break;
+      default: prec_sort_slots<16>(cand, tid, NT, M); break;
     }
     // savings of the sorted candidates, chunked over the threads
     const int per = M / NT > 0 ? M / NT : 1;
@@ -1792,15 +1850,26 @@ calc_precision_kernel(int32_t* __restrict__ b, const float* __restrict__ C, cons
       for (int q = 0; q < st; q++) cur = prec_next_bits(cur);
       mine += (double)(w[idx] * (int64_t)(cur - prec_next_bits(cur)));
     }
-    part_s[tid] = (lo < M) ? mine : 0.0;
-    __syncthreads();
-    if (tid == 0) {  // exclusive prefix over the partial sums
-      double run = 0.0;
-      for (int t = 0; t < NT; t++) { const double v = part_s[t]; part_s[t] = run; run += v; }
-      if (b_sum0 - run > target) flag_s = 2;  // every step taken and still over budget
+    // exclusive prefix of the threads' savings: a scan inside every wave, then the waves' totals (the terms are
+    // integers below 2^53, so the sums are exact in any order)
+    if (lo >= M) mine = 0.0;
+    double incl = mine;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const double up = __shfl_up(incl, off, 64);
+      if ((tid & 63) >= off) incl += up;
     }
+    if ((tid & 63) == 63) part_s[tid >> 6] = incl;   // at most 16 waves
     __syncthreads();
-    double running = b_sum0 - part_s[tid];
+    double before = 0.0, total = 0.0;
+    for (int wv = 0; wv < (NT + 63) >> 6; wv++) {
+      const double v = part_s[wv];
+      if (wv < (tid >> 6)) before += v;
+      total += v;
+    }
+    if (tid == 0 && b_sum0 - total > target) flag_s = 2;  // every step taken and still over budget
+    __syncthreads();
+    double running = b_sum0 - (before + incl - mine);
     for (int t = lo; t < hi && t < M; t++) {
       const uint64_t c = cand[t];
       if (c == 0 || !(running > target)) break;
@@ -2384,7 +2453,10 @@ int gact_calc_precision_device(int32_t* b, const float* C, const int64_t* w, int
       hipFuncSetAttribute((const void*)calc_precision_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
           hipSuccess)
     return GACT_ELAUNCH;
-  hipLaunchKernelGGL(calc_precision_kernel, dim3(1), dim3(L <= 256 ? 256 : PREC_THREADS), lds, (hipStream_t)stream, b, C, w,
+  // one thread per candidate slot up to the largest workgroup: the sort's passes are what the kernel spends its time
+  // on (120 tensors: 65.7 us with 64 threads, 25.5 with 256, 22.6 with 512; 24 tensors: 12.0 with 128, 14.1 with 256)
+  const unsigned threads = (unsigned)(M < 64 ? 64 : M > PREC_THREADS ? PREC_THREADS : M);
+  hipLaunchKernelGGL(calc_precision_kernel, dim3(1), dim3(threads), lds, (hipStream_t)stream, b, C, w,
                      (int)L, target, status);
   return launch_status();
 }
