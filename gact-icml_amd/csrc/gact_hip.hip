@@ -136,7 +136,8 @@ __device__ __forceinline__ void stream_store(V v, V* p) {
 // store the compiler emits for __builtin_nontemporal_store lets the L2 collect the lines first, which costs a float
 // write stream up to 6 % (dequantize alone, buffers cold in every cache: 4 bit 103 M elements 75.5 -> 71.3 us, 256 M
 // 183.4 -> 172.4; 8 bit 1 %; 2 bit equal; 17 M elements 1-3 % at every width; half 0-2 %), while float at 1 bit,
-// whose stream has the smallest share of reads, loses 3-4 % by it from 50 M elements on (66.3 -> 68.5 us at 103 M).
+// whose stream has the smallest share of reads, loses 3-4 % by it from 50 M elements on (66.3 -> 68.5 us at 103 M)
+// and keeps the plain nontemporal store on large tensors.
 // A window is a buffer resource over the bytes from a wave-uniform base to the end of the tensor (at most 4 GB of
 // them: offsets inside a window are 32 bit), so a store past the end of the tensor is dropped by the hardware.
 #define GACT_STORE_NT 2          /* cache-policy bits of a buffer store: 1 sc0, 2 nt, 16 sc1 */
@@ -921,7 +922,7 @@ __device__ __forceinline__ float row_bcast_at(float v, int g) {
   }
 }
 
-template <typename T, int BITS, int SGS, int PARTS = 1>
+template <typename T, int BITS, int SGS, int PARTS = 1, bool LARGE = true>
 __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ packed,
                                                 const typename Elem<T>::Stat* __restrict__ scale,
                                                 const T* __restrict__ mn, int64_t numel, int64_t N, int64_t unit,
@@ -938,7 +939,8 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
   const int64_t n_sg = (N + WPT - 1) / WPT;
   const int64_t g0 = sg0 * WPT + part * NI;   // first group of the unit
   const int rl = l & 15;  // lane within its 16-lane row
-  constexpr int POLICY = (sizeof(T) == 4 && BITS == 1) ? GACT_STORE_NT : GACT_STORE_NT_SYSTEM;
+  // float at 1 bit keeps the plain nontemporal store on large tensors (and in the batched launch)
+  constexpr int POLICY = (sizeof(T) == 4 && BITS == 1 && LARGE) ? GACT_STORE_NT : GACT_STORE_NT_SYSTEM;
   // the wave's output window starts at the first group of its first unit (a wave holds one or two units, in order)
   const int64_t window_first = wave_first(g0) * GROUP;
   const OutWindow window(out + window_first, (numel - window_first) * (int64_t)sizeof(T));
@@ -1281,8 +1283,8 @@ dequantize_kernel(const uint8_t* __restrict__ packed, const typename Elem<T>::St
   constexpr int LPU = GROUP / Elem<T>::kDqWidth;  // lanes per unit: 64 (float) or 32 (half)
   const int64_t unit = ((int64_t)xcd_tile<(uint32_t)D.run>(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x) / LPU;
   if (unit * dq_unit_groups(D, BITS, LARGE) >= N) return;
-  dequantize_unit<T, BITS, LARGE ? D.sgs_large : D.sgs, LARGE ? D.parts_large : D.parts>(packed, scale, mn, numel, N, unit,
-                                                                                       threadIdx.x % LPU, out);
+  dequantize_unit<T, BITS, LARGE ? D.sgs_large : D.sgs, LARGE ? D.parts_large : D.parts, LARGE>(packed, scale, mn, numel, N,
+                                                                                              unit, threadIdx.x % LPU, out);
 }
 
 template <typename T>
