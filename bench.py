@@ -69,17 +69,23 @@ WORKLOADS = {
     "config3-gelu": ((16384, 4096), "float16", 4, "fast", "randn", "BERT-large GELU inputs fp16, 4 bit"),
     "config3-probs": ((32, 16, 512, 512), "float16", 2, "fast", "softmax", "BERT-large attention probs fp16, 2 bit"),
     "config4": ((169343, 256), "float32", 1, "fast", "relu60", "GCN node features fp32 [169343,256], ~60% zeros, 1 bit"),
+    # the reference's own micro-benchmark (tests/test_speed.py:6-15): torch.rand [256,256,14,14] at 2 bit
+    "reference-test-speed": ((256, 256, 14, 14), "float32", 2, "fast", "rand",
+                             "the reference's tests/test_speed.py tensor: fp32 [256,256,14,14] ~U(0,1), 2 bit, stochastic rounding"),
     # not a BASELINE workload: the GELU-input tensor of config 3 as mixed-precision training on this GPU holds it
     "bf16-gelu": ((16384, 4096), "bfloat16", 4, "fast", "randn", "GELU inputs in bfloat16, 4 bit (float scale, bfloat16 min)"),
 }
 # what a default run measures besides the headline workload (config5 is the batched one)
-BASELINE_SET = ["config1", "config2", "config2-2bit", "config3-hidden", "config3-gelu", "config3-probs", "config4"]
+BASELINE_SET = ["config1", "config2", "config2-2bit", "config3-hidden", "config3-gelu", "config3-probs", "config4",
+                "reference-test-speed"]
 
 
 def make_input(torch, shape, dtype, kind, seed=0):
     g = torch.Generator(device="cuda").manual_seed(seed)
     x = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32)
-    if kind == "relu":
+    if kind == "rand":
+        x = torch.rand(shape, generator=g, device="cuda", dtype=torch.float32)
+    elif kind == "relu":
         x = torch.relu(x)
     elif kind == "relu60":
         x = torch.relu(x - 0.2533)  # P(N(0,1) < 0.2533) = 0.6
@@ -370,6 +376,31 @@ def cpu_baseline(torch, x, bits, stream, budget_s=10.0, max_elems=1 << 23):
     }
 
 
+def python_ops_us(torch, name, min_seconds):
+    """op_quantize and op_dequantize of the Python face, launched from the host one call after the other."""
+    from gact import ops
+
+    shape, dtype, bits, stream, kind, _ = WORKLOADS[name]
+    x = make_input(torch, shape, dtype, kind)
+    out = {}
+    q = ops.op_quantize(x, bits, 0, rng_stream=stream)
+    for key, fn in (("quantize", lambda: ops.op_quantize(x, bits, 0, rng_stream=stream)),
+                    ("dequantize", lambda: ops.op_dequantize(q, x.shape))):
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        calls, t0 = 0, time.perf_counter()
+        while True:
+            for _ in range(100):
+                fn()
+            torch.cuda.synchronize()
+            calls += 100
+            if time.perf_counter() - t0 >= min(min_seconds, 0.5):
+                break
+        out[key] = (time.perf_counter() - t0) / calls * 1e6
+    return out
+
+
 def compact(res):
     """The per-configuration entry of the JSON line."""
     out = {
@@ -472,6 +503,9 @@ def main():
         cached["desc"] = "config1 with one buffer set (cache-resident between steps)"
         configs["config1-cached"] = cached
         torch.cuda.empty_cache()
+        # the same tensor the way the reference's test times it: op_quantize / op_dequantize called from Python
+        # (allocations included), synchronised around each batch of calls
+        configs["reference-test-speed"]["python_ops_us"] = python_ops_us(torch, "reference-test-speed", args.min_seconds)
         line["configs"] = configs
         line["ceilings"] = run_ceilings(torch, timer, "config2")
         torch.cuda.empty_cache()
