@@ -177,7 +177,9 @@ __device__ __forceinline__ uint32_t rint_clamp0(float z) {
 // 1.5 * 2^23 + rint(y - 0.5): in that binade a float's unit in the last place is 1, the constant is even, so
 // ties go to even exactly as rint's do, and the integer sits in the low mantissa bits.  For 0 <= y < 0.5 the
 // difference lies in [-0.5, 0) (possibly rounded, which cannot take it out of that interval) and the sum rounds
-// to the constant itself: code 0, the reference's fmax.  NaN stays NaN, whose low byte is 0: code 0 as well.
+// to the constant itself: code 0, the reference's fmax.  NaN stays NaN with its payload: code 0 only where the
+// payload's low byte is 0 - true of every NaN widened from half or bfloat16 and of the NaN arithmetic generates,
+// not of any float NaN (the float path takes code_bits_of_any).
 // Two additions; the bits above the code (0x4B4...) never reach the low 8 bits a byte keeps of a code shifted
 // left by at most 7.  NOT valid for negative y (the callers' y is a sum of non-negative terms: with the group's own
 // minimum no element lies below it) and for +inf, whose bits have a zero low byte where the reference's saturated
@@ -266,7 +268,9 @@ template <> struct Elem<float> {
   __device__ static __forceinline__ uint32_t code1(const Store& st, int k, int e, float mn, float s, float u) {
     float t = st.v[k][e] - mn;
     float y = __builtin_fmaf(t, s, u);
-    return ANY ? rint_clamp0<true>(y - 0.5f) : code_bits_of(y);
+    // a NaN element keeps its payload through the subtraction and the fma, and a payload may have anything in its
+    // low byte: the clamping form (code 0 for every NaN, like the reference's fmax) rather than code_bits_of
+    return ANY ? rint_clamp0<true>(y - 0.5f) : code_bits_of_any(y);
   }
   template <bool CONST_NOISE, bool ANY>
   __device__ static __forceinline__ void codes(const Store& st, int k, float mn, float s, const float (&u)[4],
@@ -1934,7 +1938,7 @@ __device__ __forceinline__ int batch_find(const gact_batch_entry* __restrict__ t
 // (this part depends on the geometry only, not on the widths).
 __global__ void __launch_bounds__(256)
 batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int L, int64_t total_blocks,
-                  int64_t capacity, BatchWorkspace ws) {
+                  int64_t capacity, BatchWorkspace ws, int64_t* __restrict__ verdict) {
   if (blockIdx.x > 0) {
     const int64_t g = (int64_t)(blockIdx.x - 1) * blockDim.x + threadIdx.x;
     if (g < total_blocks) ws.block_tensor[g] = batch_find(table, L, g);
@@ -1975,8 +1979,13 @@ batch_plan_kernel(gact_batch_entry* table, const int32_t* __restrict__ bits, int
     for (int k = 0; k < 4; k++) cnt[k] += __shfl_xor(cnt[k], off, 64);
   }
   if (lane == 0) {
+    const int64_t ok = (!bad && base <= capacity) ? 1 : 0;
     ws.hdr->need = base;
-    ws.hdr->ok = (!bad && base <= capacity) ? 1 : 0;
+    ws.hdr->ok = ok;
+    if (verdict) {   // the same two words where the caller can see them
+      verdict[0] = base;
+      verdict[1] = ok;
+    }
 #pragma unroll
     for (int k = 0; k < 4; k++) ws.hdr->tensors_at[k] = cnt[k];
   }
@@ -2053,6 +2062,9 @@ namespace {
 
 inline bool valid_bits(int bits) { return bits == 1 || bits == 2 || bits == 4 || bits == 8; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+// hipGetLastError returns and clears the thread's last error, which may be one an earlier call of the caller's left
+// behind: an entry point clears it before its first launch (fresh_launch) and reports what its own launches left.
+inline void fresh_launch() { (void)hipGetLastError(); }
 inline int launch_status() { return hipGetLastError() == hipSuccess ? GACT_OK : GACT_ELAUNCH; }
 
 // one 16-lane row per unit of work (a super-group for quantize / dequantize, 8 groups for minimax);
@@ -2291,6 +2303,7 @@ int gact_minimax(const void* data, int dtype, int64_t N, int64_t D, void* mn, vo
   if (N == 0) return GACT_OK;
   if (!data || !mn || !mx) return GACT_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  fresh_launch();
   if (D == GROUP && aligned16(data)) {
     dim3 grid, block;
     row_grid((N + MINIMAX_ROW_GROUPS - 1) / MINIMAX_ROW_GROUPS, &grid, &block, MINIMAX_THREADS);
@@ -2317,6 +2330,7 @@ int gact_pack(const void* data, const void* mn, const void* mx, int dtype, int b
   if (!data || !mn || !mx || !packed || !scale) return GACT_EINVAL;
   if (noise_mode == GACT_NOISE_INJECT && !noise) return GACT_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  fresh_launch();
   if (G == 1 && D == GROUP && aligned16(data) && aligned16(packed) && (noise_mode != GACT_NOISE_INJECT || aligned16(noise))) {
     // the fused row kernel with min/max taken from the caller
     if (dtype == GACT_F32)
@@ -2343,6 +2357,7 @@ int gact_unpack(const void* packed, int bits, const void* scale, const void* mn,
   if (N * G * D == 0) return GACT_OK;
   if (!packed || !scale || !mn || !out) return GACT_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  fresh_launch();
   if (G == 1 && D == GROUP && aligned16(out) && aligned16(packed)) {
     if (dtype == GACT_F32)
       return dispatch_dequantize<float>(bits, (const uint8_t*)packed, (const float*)scale, (const float*)mn, N * GROUP, N, (float*)out, s);
@@ -2366,6 +2381,7 @@ int gact_quantize_seeded(const void* x, int dtype, int64_t numel, int bits, int 
   if (reinterpret_cast<uintptr_t>(seed_add) & 7u) return GACT_EALIGN;
   const int64_t N = (numel + GROUP - 1) / GROUP;
   hipStream_t s = (hipStream_t)stream;
+  fresh_launch();
   const SeedArg sa{seed, seed_add};
   if (dtype == GACT_F32)
     return dispatch_quantize<float, false>(bits, (const float*)x, numel, N, (uint8_t*)packed, (float*)scale, (float*)mn, (float*)mx, noise_mode, sa, noise, s);
@@ -2388,6 +2404,7 @@ int gact_dequantize(const void* packed, int bits, const void* scale, const void*
   if (!aligned16(out) || !aligned16(packed)) return GACT_EALIGN;
   const int64_t N = (numel + GROUP - 1) / GROUP;
   hipStream_t s = (hipStream_t)stream;
+  fresh_launch();
   if (dtype == GACT_F32)
     return dispatch_dequantize<float>(bits, (const uint8_t*)packed, (const float*)scale, (const float*)mn, numel, N, (float*)out, s);
   if (dtype == GACT_BF16)
@@ -2400,6 +2417,7 @@ int gact_mask_pack(const uint8_t* data, int64_t n, int32_t* mask, void* stream) 
   if (n == 0) return GACT_OK;
   if (!data || !mask) return GACT_EINVAL;
   if (!aligned16(data)) return GACT_EALIGN;
+  fresh_launch();
   const int64_t pairs = (n / 512 + 1) / 2;  // pairs of full blocks
   const int64_t waves = (pairs + MASK_PAIRS - 1) / MASK_PAIRS + 1;  // plus the wave that takes the partial block
   hipLaunchKernelGGL(mask_pack_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, (hipStream_t)stream, data, n, mask);
@@ -2411,6 +2429,7 @@ int gact_mask_unpack(const int32_t* mask, int64_t n, uint8_t* out, void* stream)
   if (n == 0) return GACT_OK;
   if (!mask || !out) return GACT_EINVAL;
   if (!aligned16(out)) return GACT_EALIGN;
+  fresh_launch();
   const int64_t blocks = n / 512 + 1;  // the partial block included
   const int64_t waves = (blocks + MASK_STEPS * 4 - 1) / (MASK_STEPS * 4);
   hipLaunchKernelGGL(mask_unpack_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, (hipStream_t)stream, mask, n, out);
@@ -2448,6 +2467,7 @@ int gact_calc_precision_device(int32_t* b, const float* C, const int64_t* w, int
   if (L > PREC_MAX_L) return GACT_ESHAPE;
   if (L == 0) return GACT_OK;
   if (!b || !C || !w) return GACT_EINVAL;
+  fresh_launch();
   int64_t M = 4;
   while (M < 4 * L) M <<= 1;
   const size_t lds = (size_t)M * sizeof(uint64_t);
@@ -2470,10 +2490,10 @@ int64_t gact_batch_workspace_bytes(int64_t L, int64_t total_blocks) {
 
 namespace {
 int batch_plan_on(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks, int64_t capacity,
-                  void* workspace, hipStream_t s) {
+                  void* workspace, int64_t* verdict, hipStream_t s) {
   const BatchWorkspace ws = batch_workspace(workspace);
   hipLaunchKernelGGL(batch_plan_kernel, dim3((unsigned)(1 + (total_blocks + 255) / 256)), dim3(256), 0, s, table, bits, (int)L,
-                     total_blocks, capacity, ws);
+                     total_blocks, capacity, ws, verdict);
   return launch_status();
 }
 
@@ -2512,7 +2532,8 @@ int gact_batch_plan(gact_batch_entry* table, const int32_t* bits, int64_t L, int
   if (!workspace) return GACT_EINVAL;
   if (!aligned16(workspace)) return GACT_EALIGN;
   if (L > 0 && (!table || !bits)) return GACT_EINVAL;
-  return batch_plan_on(table, bits, L, total_blocks, capacity, workspace, (hipStream_t)stream);
+  fresh_launch();
+  return batch_plan_on(table, bits, L, total_blocks, capacity, workspace, nullptr, (hipStream_t)stream);
 }
 
 int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
@@ -2526,6 +2547,7 @@ int gact_quantize_batched(const gact_batch_entry* table, const int32_t* bits, in
   if (L == 0 || total_blocks == 0) return GACT_OK;
   if (!table || !bits || !workspace || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena) || !aligned16(workspace)) return GACT_EALIGN;
+  fresh_launch();
   return quantize_batched_on(table, bits, total_blocks, noise_mode, dtypes, const_cast<void*>(workspace), packed_arena,
                              scale_arena, min_arena, (hipStream_t)stream);
 }
@@ -2537,6 +2559,7 @@ int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, 
   if (L == 0 || total_blocks == 0) return GACT_OK;
   if (!table || !bits || !workspace || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena) || !aligned16(workspace)) return GACT_EALIGN;
+  fresh_launch();
   const dim3 grid((unsigned)(2 * total_blocks)), block(256);
   hipLaunchKernelGGL(dequantize_batched_kernel, grid, block, 0, (hipStream_t)stream, table, bits,
                      batch_workspace(const_cast<void*>(workspace)), (const uint8_t*)packed_arena,
@@ -2549,7 +2572,9 @@ int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, 
 // of the library's own.  Every GPU the library runs on holds its own copy of the array, at its own address,
 // until the process ends; the address is looked up once per device (the array's name is only a host-side
 // handle) and that pointer is what the kernels get.  Calls on one GPU share the array: they must not overlap.
-// Nothing in it has to start at zero - the plan kernels write every field the work kernels read.
+// Nothing in it has to start at zero - the plan kernel writes every field the work kernels read, the verdict
+// (`ok`) included, on every call: a void plan left behind by an earlier call cannot leak into the next one.
+// The verdict of a call is also written to the caller's `verdict` words, since the array itself is out of reach.
 // ------------------------------------------------------------------------------------------------
 #define GACT_STATIC_MAX_BLOCKS 262144
 #define GACT_STATIC_WORKSPACE_BYTES (256 + GACT_STATIC_MAX_BLOCKS * 4)
@@ -2576,7 +2601,7 @@ int static_workspace(void** out) {
 
 int gact_quantize_batched_static(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
                                  int64_t capacity, int noise_mode, int dtypes, void* packed_arena, void* scale_arena,
-                                 void* min_arena, void* stream) {
+                                 void* min_arena, int64_t* verdict, void* stream) {
   if (!batched_args_ok(L, total_blocks) || capacity < 0) return GACT_EINVAL;
   if (noise_mode != GACT_NOISE_CONST && noise_mode != GACT_NOISE_REF && noise_mode != GACT_NOISE_FAST) return GACT_EINVAL;
   if (dtypes < 0 || dtypes > GACT_DTYPES_ALL) return GACT_EINVAL;
@@ -2585,11 +2610,13 @@ int gact_quantize_batched_static(gact_batch_entry* table, const int32_t* bits, i
   if (L == 0 || total_blocks == 0) return GACT_OK;
   if (!table || !bits || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena)) return GACT_EALIGN;
+  if (reinterpret_cast<uintptr_t>(verdict) & 7u) return GACT_EALIGN;
   void* ws = nullptr;
   const int rc = static_workspace(&ws);
   if (rc != GACT_OK) return rc;
   hipStream_t s = (hipStream_t)stream;
-  const int planned = batch_plan_on(table, bits, L, total_blocks, capacity, ws, s);
+  fresh_launch();
+  const int planned = batch_plan_on(table, bits, L, total_blocks, capacity, ws, verdict, s);
   if (planned != GACT_OK) return planned;
   return quantize_batched_on(table, bits, total_blocks, noise_mode, dtypes, ws, packed_arena, scale_arena, min_arena, s);
 }

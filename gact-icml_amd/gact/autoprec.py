@@ -14,10 +14,12 @@ import numpy as np
 import torch
 import torch.nn as nn
 
+from .conf import config
 from .cpp_extension import calc_precision as ext_calc_precision
 from .utils import exp_recorder
 
 SENSITIVITY_CAP = 1e10
+DEVICE_CALC_PRECISION_MAX_TENSORS = 4096     # what one launch of the device allocation takes
 
 
 def _seed_everything(seed):
@@ -139,11 +141,16 @@ class AutoPrecision:
             # reads every sensitivity back as soon as its three passes are queued); one read-back at the end
             layers = list(self.quantizer.bits)
             sens = [self._sensitivity_of(l, backprop) for l in layers]
-            if sens:
-                values = torch.stack([v.double() for v in sens]).tolist()
-                for l, v in zip(layers, values):
-                    self.C[l] = SENSITIVITY_CAP if v >= SENSITIVITY_CAP else v
-            self.refresh_bits()
+            if sens and self._allocates_on_device(layers, sens):
+                # the sensitivities never visit the host before the allocation: the greedy runs on the GPU
+                # behind the probes, and widths and sensitivities come back in one copy afterwards
+                self.refresh_bits_on_device(torch.stack(sens).float())
+            else:
+                if sens:
+                    values = torch.stack([v.double() for v in sens]).tolist()
+                    for l, v in zip(layers, values):
+                        self.C[l] = SENSITIVITY_CAP if v >= SENSITIVITY_CAP else v
+                self.refresh_bits()
 
         if adapting and self.debug:
             # the variance model against a measurement: gradient at the allocated widths vs uncompressed
@@ -171,6 +178,12 @@ class AutoPrecision:
 
         self.iter += 1
 
+    def _allocates_on_device(self, layers, sens):
+        """config.device_calc_precision, and the probes cover the dims table in its order on a GPU (they do
+        whenever the quantizer's tables come from one first iteration) with few enough tensors for one launch."""
+        return (config.device_calc_precision and sens[0].is_cuda and layers == list(self.dims)
+                and len(layers) <= DEVICE_CALC_PRECISION_MAX_TENSORS)
+
     def refresh_bits(self):
         """Greedy allocation from the current sensitivities: every tensor starts at max_bits, tensors are
         listed in the order of the dims table (gact/gact/autoprec.py:188-209)."""
@@ -180,7 +193,29 @@ class AutoPrecision:
                                                    torch.tensor([self.C[l] for l in order], dtype=torch.float),
                                                    torch.tensor([self.dims[l] for l in order], dtype=torch.int64),
                                                    self.total_bits)
-        for l, b in zip(order, chosen.tolist()):
+        self._adopt_bits(order, chosen.tolist())
+
+    def refresh_bits_on_device(self, C_dev):
+        """The same allocation (calc_precision.cc:66-118) by the device kernel, from sensitivities that are still
+        on the GPU: float32[len(dims)] in the order of the dims table.  One read-back, after the launch, brings
+        the widths (and the sensitivities, for the log and the variance model) to the host."""
+        order = list(self.dims)
+        dev = C_dev.device
+        start = torch.full((len(order),), self.max_bits, dtype=torch.int32, device=dev)
+        if getattr(self, "_dims_dev", None) is None or self._dims_dev.device != dev or self._dims_dev.numel() != len(order):
+            self._dims_dev = torch.tensor([self.dims[l] for l in order], dtype=torch.int64, device=dev)
+        status = torch.zeros((1,), dtype=torch.int32, device=dev)
+        ext_calc_precision.calc_precision_device(start, C_dev.contiguous(), self._dims_dev, self.total_bits, status)
+        back = torch.cat([start.double(), status.double(), C_dev.double()]).tolist()
+        L = len(order)
+        if int(back[L]) != 0:
+            raise RuntimeError("calc_precision on the device failed with status %d" % int(back[L]))
+        for l, v in zip(order, back[L + 1:]):
+            self.C[l] = SENSITIVITY_CAP if v >= SENSITIVITY_CAP else v
+        self._adopt_bits(order, [int(b) for b in back[:L]])
+
+    def _adopt_bits(self, order, chosen):
+        for l, b in zip(order, chosen):
             self.bits[l] = b
         self.quantizer.bits = self.bits.copy()
 

@@ -2,10 +2,11 @@
 
 The reference quantizes one tensor per call (gact/gact/quantizer.py:95-142) and computes the widths on
 the host (gact/gact/autoprec.py:188-209).  Here ``calc_precision_device`` leaves the widths in device
-memory, a planning step (two small kernels) turns them into packed-arena offsets and into a list of the
-grid's blocks sorted by width, and the batched kernels then quantize (one launch per width, each over its
-own blocks) or dequantize (one launch) every tensor at its own width.  Nothing is read back to the host;
-the results are identical to calling ``op_quantize`` / ``op_dequantize`` tensor by tensor.
+memory and one small planning launch turns them into packed-arena offsets (and says which tensor every
+block of the grid belongs to); the batched kernels then quantize (one launch per element type over all
+blocks, a block's width selecting its code path) or dequantize (one launch for every type and width)
+every tensor at its own width.  Nothing is read back to the host; the results are identical to calling
+``op_quantize`` / ``op_dequantize`` tensor by tensor.
 
 Grid layout: a block owns 128 groups of 256 elements whatever the width, so the grid
 (sum over tensors of ceil(N_i/128) blocks) is known on the host without knowing the widths.
@@ -101,7 +102,7 @@ class BatchedQuantizer:
         return sum(self.numels) + 768 * self.L + 256
 
     def new_workspace(self):
-        """Device memory a plan of this geometry fills (header, block -> tensor map, blocks sorted by kind)."""
+        """Device memory a plan of this geometry fills: a 256-byte header (the verdict) and the block -> tensor map."""
         return torch.empty((self.workspace_bytes,), dtype=torch.uint8, device=self.device)
 
     def plan_ok(self, workspace):

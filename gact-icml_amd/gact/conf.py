@@ -25,6 +25,11 @@ class QuantizationConfig:
         self.log_interval = -1      # < 0 disables logging
         self.debug = False
 
+        # Run the greedy allocation on the GPU (not in the reference): the sensitivities of an adaptation stay in
+        # device memory, calc_precision runs there behind the probes, and one copy brings the widths back.
+        # Same widths as the host routine.
+        self.device_calc_precision = False
+
         # ---- memory management ----
         self.swap = False
         self.prefetch = False

@@ -15,7 +15,7 @@ F32, F16, BF16 = 0, 1, 2
 NOISE_CONST, NOISE_INJECT, NOISE_REF, NOISE_FAST = 0, 1, 2, 3
 NOISE_MODES = {"deterministic": NOISE_CONST, "inject": NOISE_INJECT, "reference": NOISE_REF, "fast": NOISE_FAST}
 GROUP = 256
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class BatchEntry(ctypes.Structure):
@@ -54,7 +54,7 @@ SIGNATURES = {
     "gact_batch_plan": (_i32, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
     "gact_quantize_batched": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "gact_dequantize_batched": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
-    "gact_quantize_batched_static": (_i32, [_vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp]),
+    "gact_quantize_batched_static": (_i32, [_vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
 }
 
 

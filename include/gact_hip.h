@@ -17,7 +17,7 @@
 extern "C" {
 #endif
 
-#define GACT_ABI_VERSION 5
+#define GACT_ABI_VERSION 6
 
 /* element types of activations, min, max and scale */
 #define GACT_F32 0
@@ -157,14 +157,17 @@ int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, 
  * caller brings: nothing is allocated, by the library or on its behalf.  No counterpart in the reference; it
  * is for callers that cannot allocate - code under HIP graph capture, tight serving loops, harnesses that
  * forbid it.  Same results as the two calls it stands for (packed_offset of every table entry is filled, the
- * arenas are written); the plan's verdict stays in the library's array, so size the arena for the worst case
- * or check the widths beforehand.  Limit: total_blocks <= 262144 (33.5 M groups, 8.6 G elements),
+ * arenas are written).  The plan's verdict lives in the library's array, out of the caller's reach, so the plan
+ * also writes it to `verdict` (two int64 in device memory, 8-byte aligned; may be null): [0] the arena bytes the
+ * table needs, [1] 1 when the launch went ahead, 0 when it was void (a width outside {1,2,4,8}, an unknown
+ * element type, or [0] > capacity: the arenas are then left untouched).  Read it whenever the caller may
+ * synchronise.  Limit: total_blocks <= 262144 (33.5 M groups, 8.6 G elements),
  * GACT_ELIMIT beyond.  All calls on one GPU share the array: calls that overlap on one GPU (two streams, two
  * threads) race, the caller serialises them.  The first call on a GPU looks the array's address up; make it
  * outside a stream capture.  Dequantize with gact_batch_plan + gact_dequantize_batched as usual. */
 int gact_quantize_batched_static(gact_batch_entry* table, const int32_t* bits, int64_t L, int64_t total_blocks,
                                  int64_t capacity, int noise_mode, int dtypes, void* packed_arena,
-                                 void* scale_arena, void* min_arena, void* stream);
+                                 void* scale_arena, void* min_arena, int64_t* verdict, void* stream);
 
 #ifdef __cplusplus
 }

@@ -111,9 +111,9 @@ def test_hooks_on_hip_kernels_equal_hooks_on_the_cpu_oracle(monkeypatch):
         assert torch.allclose(g_hip, g_cpu, rtol=1e-4, atol=1e-7)
 
 
-def train(swap, steps=6):
-    vars(config).update(dict(compress_activation=True, auto_prec=True, bit=4, swap=swap, prefetch=swap,
-                             adapt_interval=4, max_bit=32, log_interval=-1))
+def train(swap, steps=6, adapt_interval=4, max_bit=32, bit=4):
+    vars(config).update(dict(compress_activation=True, auto_prec=True, bit=bit, swap=swap, prefetch=swap,
+                             adapt_interval=adapt_interval, max_bit=max_bit, log_interval=-1))
     net = make_net()
     net.eval()      # no dropout / batch statistics: the run must be reproducible bit for bit
     opt = torch.optim.SGD(net.parameters(), lr=0.05)
@@ -262,3 +262,120 @@ def test_saved_bool_masks_are_packed_to_one_bit_losslessly(monkeypatch):
     assert q.quantize(small) == (False, small) or q.quantize(small)[1] is small
     config.compress_bool_masks = False
     assert q.quantize(m)[0] is False
+
+
+class TwoReaders(nn.Module):
+    """One activation saved for backward by two operators: both linear layers keep `h` as their input."""
+
+    def __init__(self):
+        super().__init__()
+        torch.manual_seed(0)
+        self.stem = nn.Linear(64, 128)
+        self.left, self.right = nn.Linear(128, 32), nn.Linear(128, 32)
+
+    def forward(self, x):
+        h = torch.relu(self.stem(x))
+        return self.left(h) + self.right(h)
+
+
+def test_check_dup_compresses_a_twice_saved_activation_once(monkeypatch):
+    """quantizer.py:85-93,106-112,138-141 of the reference: with config.check_dup the key of a saved tensor is its
+    address, a strided sample and its sum, a second save under the same key adds a consumer instead of new
+    codes, and the codes are dropped when the last consumer has read them."""
+    import gact.quantizer as quantizer_mod
+
+    real_q = quantizer_mod.op_quantize
+    launches = []
+
+    def counting_q(t, *a, **k):
+        launches.append((t.data_ptr(), tuple(t.shape)))
+        return real_q(t, *a, **k)
+
+    monkeypatch.setattr(quantizer_mod, "op_quantize", counting_q)
+    torch.manual_seed(5)
+    x = torch.randn(48, 4, 64, device="cuda")       # rank 3: the input is compressed too
+    target = torch.randn(48, 4, 32, device="cuda")
+    results = {}
+    for dup in (False, True):
+        vars(config).update(dict(compress_activation=True, auto_prec=False, bit=4, swap=False, prefetch=False,
+                                 check_dup=dup, rng_stream="deterministic"))
+        net = TwoReaders().cuda()
+        ctl = Controller(net)
+        launches.clear()
+        with ctl:
+            loss = nn.functional.mse_loss(net(x), target)
+            held = {k: v[1] for k, v in ctl.quantizer.ptr_qtensor_map.items()}
+            saves = ctl.quantizer.tid
+            loss.backward()
+        results[dup] = (list(launches), held, saves, dict(ctl.quantizer.ptr_qtensor_map),
+                        torch.cat([p.grad.ravel() for p in net.parameters()]))
+    plain, deduped = results[False], results[True]
+    assert plain[2] == deduped[2] >= 3                  # the hooks saw the same saves either way
+    assert len(plain[0]) == plain[2]                    # one launch per save without check_dup
+    # the key is the address, a strided sample and the sum, not the shape: h is saved by relu as [48,4,128] and by
+    # both readers as [192,128], three saves of one buffer
+    addresses = [p for p, _ in plain[0]]
+    shared = [p for p in set(addresses) if addresses.count(p) > 1]
+    assert len(shared) == 1 and addresses.count(shared[0]) == 3
+    # with check_dup: one launch per distinct buffer, the shared one held for all of its consumers
+    assert len(deduped[0]) == len(set(addresses)) == deduped[2] - 2
+    assert sorted(deduped[1].values()) == [1] * (len(set(addresses)) - 1) + [3]
+    assert plain[3] == {} and deduped[3] == {}          # every compressed copy was released by the backward pass
+    assert torch.equal(plain[4], deduped[4])            # deterministic rounding: the very same gradients
+
+
+def test_device_calc_precision_gives_the_host_tables(monkeypatch):
+    """config.device_calc_precision: the sensitivities stay on the GPU, the greedy of calc_precision.cc:66-118 runs
+    there, and the tables (autoprec.py:188-209 of the reference) equal the host routine's on the same
+    sensitivities, adaptation after adaptation, from max_bit 32 and from 8."""
+    from gact.autoprec import AutoPrecision
+
+    seen = []
+    on_device = AutoPrecision.refresh_bits_on_device
+
+    def both(self, C_dev):
+        on_device(self, C_dev)
+        device_bits, device_C = dict(self.bits), dict(self.C)
+        assert self.quantizer.bits == device_bits
+        self.refresh_bits()                     # the host routine on the sensitivities that came back
+        assert self.C == device_C
+        seen.append((device_bits, dict(self.bits)))
+
+    monkeypatch.setattr(AutoPrecision, "refresh_bits_on_device", both)
+    for max_bit, avg in ((32, 4), (8, 2), (32, 3)):
+        before = len(seen)
+        vars(config).update(dict(device_calc_precision=True))
+        losses, bits = train(swap=False, steps=6, adapt_interval=2, max_bit=max_bit, bit=avg)
+        assert len(seen) - before == 3          # adaptations at iterations 0, 2, 4
+        for device_bits, host_bits in seen[before:]:
+            assert device_bits == host_bits and len(device_bits) >= 4
+            assert set(device_bits.values()) <= {1, 2, 4, 8, 32}
+        assert bits == seen[-1][0]
+        assert all(l == l for l in losses)
+
+
+def test_device_calc_precision_on_ties_zero_and_capped_sensitivities():
+    from gact.autoprec import AutoPrecision, SENSITIVITY_CAP
+
+    class Tables:
+        bits = {}
+
+    dims = {i: n for i, n in enumerate([4096, 4096, 4096, 100, 100, 65536, 65536, 7, 300000, 300000])}
+    cases = [[1.0] * 10, [0.0] * 10, [SENSITIVITY_CAP] * 5 + [0.0] * 5,
+             [3.0, 3.0, 3.0, 1e-30, 1e-30, 7.5, 7.5, 1e10, 0.5, 0.5], [float(i % 3) for i in range(10)]]
+    for max_bit, avg in ((32, 4), (8, 2), (8, 1), (32, 8)):
+        for C in cases:
+            tables = []
+            for device in (False, True):
+                ap = AutoPrecision(None, Tables(), avg, max_bit, "/tmp", 1, -1)
+                ap.quantizer.dims = dict(dims)
+                ap.init_from_dims()
+                if device:
+                    ap.refresh_bits_on_device(torch.tensor(C, dtype=torch.float32, device="cuda"))
+                    assert [ap.C[l] for l in dims] == [float(torch.tensor(c, dtype=torch.float32)) for c in C]
+                else:
+                    ap.C = {l: c for l, c in zip(dims, C)}
+                    ap.refresh_bits()
+                tables.append(dict(ap.bits))
+                assert ap.quantizer.bits == ap.bits
+            assert tables[0] == tables[1], (max_bit, avg, C, tables)

@@ -144,6 +144,28 @@ def test_edge_groups(dtype, bits):
         np.testing.assert_array_equal(out[m], want[m])
 
 
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+def test_nan_payloads_give_code_zero_like_the_reference(bits):
+    """quantization_cuda_kernel.cu:66: fmax(NaN, 0) is 0 whatever the NaN's bits.  float NaNs other than the one
+    arithmetic generates (0x7fc00000) keep their payload through the kernel's arithmetic; their low byte must
+    not leak into the code, nor into the neighbouring groups' fields of the same byte."""
+    torch.manual_seed(9)
+    x = torch.randn(32, 256)
+    raw = x.view(torch.int32)
+    patterns = [0x7fc00001, 0x7fffffff, 0x7fc000ff, 0x7fe0a5c3, -0x003fff01]   # the last: 0xffc000ff, a negative NaN
+    for g in range(0, 32, 3):
+        for k, pat in enumerate(patterns):
+            raw[g, (37 * g + 50 * k) % 256] = pat
+    assert torch.isnan(x).sum() == 11 * len(patterns)
+    noise = torch.rand(x.shape)
+    for mode in ("deterministic", "reference", "fast"):
+        q, ref = check_quantize(x, bits, mode, seed=4)
+        out = ops.op_dequantize(q, x.shape).cpu().numpy()
+        want = oracle.op_dequantize(ref, x.shape)
+        np.testing.assert_array_equal(out, want)       # code 0 dequantizes to the group's min: no NaN comes back
+    check_quantize(x, bits, "inject", seed=0, noise=noise)
+
+
 def test_config1_full_size_deterministic():
     # benchmark workload config 1: fp32 [4096,1024] ~ N(0,1), seed 0, 2 bit, deterministic rounding
     torch.manual_seed(0)

@@ -42,7 +42,7 @@ def test_struct_layout_matches_the_header():
 
 def test_status_codes_and_sizes():
     L = _abi.lib()
-    assert L.gact_abi_version() == 5
+    assert L.gact_abi_version() == 6
     assert L.gact_strerror(0) == b"ok"
     for code in (-1, -2, -3, -4, -5):
         assert L.gact_strerror(code) not in (b"ok", b"unknown error")
@@ -77,7 +77,7 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     assert L.gact_batch_plan(16, 16, 3, 3, 100, None, None) == -1                                # no workspace
     # header (32 int64) + one int32 per block, in whole 16-byte pieces
     assert L.gact_batch_workspace_bytes(3, 5) == 256 + 2 * 16
-    assert L.gact_quantize_batched_static(16, 16, 10, 262145, 1 << 20, 3, 0, 16, 16, 16, None) == -6   # beyond its array
+    assert L.gact_quantize_batched_static(16, 16, 10, 262145, 1 << 20, 3, 0, 16, 16, 16, None, None) == -6   # beyond its array
     assert L.gact_batch_workspace_bytes(-1, 5) == -1
     assert L.gact_quantize(16, 3, 256, 4, 0, 0, None, 16, 16, 16, None, None) == -1               # element type
     assert L.gact_quantize(0, 2, 256, 4, 0, 0, None, 16, 16, 16, None, None) == -1                # bfloat16, null data
