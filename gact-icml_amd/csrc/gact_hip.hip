@@ -7,9 +7,9 @@
 // 8i + 128m - so every load instruction of a row reads 256 contiguous bytes.  Per-group reductions are
 // four row_ror DPP steps that never leave the row, and - because the reference packs the SAME column of
 // 8/bits consecutive groups into one byte - the lane that owns a column owns every code of that byte:
-// packing needs no cross-lane traffic at all.  One Philox block feeds 8 consecutive columns - a half
-// chunk, or the float chunks of a pair of neighbouring lanes (which swap the halves they need) - and, mirrored,
-// the 8 columns half a group further on, which the same lane owns.
+// packing needs no cross-lane traffic at all.  One Philox block feeds 8 consecutive columns of two consecutive
+// groups - a half chunk, or the float chunks of a pair of neighbouring lanes (which swap the words they need) -
+// and, mirrored, the 8 columns half a group further on, which the same lane owns.
 //
 // Dequantize has no reduction, so a unit of 4 or 8 consecutive groups goes to a whole wave (float: lane l owns
 // columns 4l .. 4l+3) or half a wave (half: 8l .. 8l+7): one 16-byte store per lane and group, every store
@@ -104,9 +104,15 @@ __device__ __forceinline__ void philox4x32(uint32_t c0, uint32_t c1, uint32_t c2
 __device__ __forceinline__ float curand_uniform_map(uint32_t x) {
   return __builtin_fmaf((float)x, 0x1p-32f, 0x1p-33f);
 }
-// 16-bit noise of the fast stream: (h + 0.5) * 2^-16, exact in float.
-__device__ __forceinline__ float fast_uniform_map(uint32_t h) {
-  return __builtin_fmaf((float)h, 0x1p-16f, 0x1p-17f);
+// 8-bit centred noise of the fast stream from byte B of a Philox word: (2h - 255) / 512 = (h + 0.5) / 256 - 1/2,
+// exact in float (v_cvt_f32_ubyteB and one fma).
+template <int B>
+__device__ __forceinline__ float fast_centred_map(uint32_t w) {
+  return __builtin_fmaf((float)((w >> (8 * B)) & 0xffu), 0x1p-8f, -255.0f / 512.0f);
+}
+__device__ __forceinline__ float fast_centred_map(uint32_t w, int b) {
+  return (b & 2) ? ((b & 1) ? fast_centred_map<3>(w) : fast_centred_map<2>(w))
+                 : ((b & 1) ? fast_centred_map<1>(w) : fast_centred_map<0>(w));
 }
 
 // Activations and codes are touched exactly once per kernel: load and store them with the streaming
@@ -197,6 +203,11 @@ __device__ __forceinline__ uint32_t clamp_code_bits(float w) {
   return __builtin_bit_cast(uint32_t, c);
 }
 __device__ __forceinline__ uint32_t code_bits_of_any(float y) { return clamp_code_bits(y + 8388607.5f); }
+// The fast stream adds a centred draw, so its sum z already is the reference's y - 0.5 and the code is rint(max(z, 0)):
+// one addition (z > -0.5 with the group's own minimum, so z + 1.5 * 2^23 rounds to 1.5 * 2^23 + rint(z), -0 included),
+// or the clamping form for any z.
+__device__ __forceinline__ uint32_t centred_code_bits_of(float z) { return __builtin_bit_cast(uint32_t, z + 12582912.0f); }
+__device__ __forceinline__ uint32_t centred_code_bits_of_any(float z) { return clamp_code_bits(z + 8388608.0f); }
 
 // Correctly rounded c / s from the correctly rounded reciprocal r = RN(1/s) (Markstein): q = RN(c*r),
 // e = c - s*q exactly (one FMA), result RN(q + e*r).  Valid for finite nonzero s with a normal quotient;
@@ -264,19 +275,22 @@ template <> struct Elem<float> {
   // code = rint(max(fma(x - mn, s, u) - 0.5, 0)).  ANY = true: min and scale may be anything (the pack entry
   // point), the code is converted as the reference converts it; ANY = false: they are the group's own, the
   // sum stays below 2^bits + 1 and the code is read off the float (code_bits_of: its low 8 bits count)
-  template <bool ANY>
+  // CENTRED: u is a centred draw of the fast stream (the - 0.5 is in it)
+  template <bool ANY, bool CENTRED = false>
   __device__ static __forceinline__ uint32_t code1(const Store& st, int k, int e, float mn, float s, float u) {
     float t = st.v[k][e] - mn;
     float y = __builtin_fmaf(t, s, u);
     // a NaN element keeps its payload through the subtraction and the fma, and a payload may have anything in its
     // low byte: the clamping form (code 0 for every NaN, like the reference's fmax) rather than code_bits_of
+    if (CENTRED) return ANY ? rint_clamp0<true>(y) : centred_code_bits_of_any(y);
     return ANY ? rint_clamp0<true>(y - 0.5f) : code_bits_of_any(y);
   }
-  template <bool CONST_NOISE, bool ANY>
+  // NEG (with CENTRED): the chunk takes the mirrored draws, -u (the negation folds into the fma)
+  template <bool CONST_NOISE, bool ANY, bool CENTRED = false, bool NEG = false>
   __device__ static __forceinline__ void codes(const Store& st, int k, float mn, float s, const float (&u)[4],
                                                uint32_t (&c)[4]) {
 #pragma unroll
-    for (int e = 0; e < 4; e++) c[e] = code1<ANY>(st, k, e, mn, s, u[e]);
+    for (int e = 0; e < 4; e++) c[e] = code1<ANY, CENTRED>(st, k, e, mn, s, NEG ? -u[e] : u[e]);
   }
   // a float scale is never infinite (the denominator is at least 2e-6) and with the group's own min and max the
   // sum stays finite: nothing to repair
@@ -391,19 +405,31 @@ template <> struct Elem<f16> {
     asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(y) : "v"(p), "v"(u));
     return y;
   }
+  // float(p) - u: the same instruction with the addend's sign flipped
+  __device__ static __forceinline__ float widen_sub_lo(f16x2 p, float u) {
+    float y;
+    asm("v_fma_mix_f32 %0, %1, 1.0, -%2 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(y) : "v"(p), "v"(u));
+    return y;
+  }
+  __device__ static __forceinline__ float widen_sub_hi(f16x2 p, float u) {
+    float y;
+    asm("v_fma_mix_f32 %0, %1, 1.0, -%2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(y) : "v"(p), "v"(u));
+    return y;
+  }
   // half subtraction and half product (each rounded to half), then float: y = float(p) + u,
   // code = rint(max(y - 0.5, 0)).  |y| <= 65505 or y is infinite or NaN whatever min and scale are, so the
   // code is always read off the float.  ANY = true (min and scale from the caller): y may be negative or +inf,
   // the clamping form takes both.  ANY = false: y >= 0, and where it is +inf (the scale overflowed to inf)
   // the caller repairs the group afterwards.
-  template <bool ANY>
+  template <bool ANY, bool CENTRED = false>
   __device__ static __forceinline__ uint32_t code1(const Store& st, int k, int e, f16 mn, f16 s, float u) {
     f16 t = st.v[k][e >> 1][e & 1] - mn;
     f16 p = t * s;
     float y = (float)p + u;
+    if (CENTRED) return ANY ? centred_code_bits_of_any(y) : centred_code_bits_of(y);
     return ANY ? code_bits_of_any(y) : code_bits_of(y);
   }
-  template <bool CONST_NOISE, bool ANY>
+  template <bool CONST_NOISE, bool ANY, bool CENTRED = false, bool NEG = false>
   __device__ static __forceinline__ void codes(const Store& st, int k, f16 mn, f16 s, const float (&u)[8],
                                                uint32_t (&c)[8]) {
     const f16x2 mn2 = {mn, mn}, s2 = {s, s};
@@ -411,7 +437,13 @@ template <> struct Elem<f16> {
     for (int j = 0; j < 4; j++) {
       f16x2 t = st.v[k][j] - mn2;
       f16x2 p = t * s2;
-      if (CONST_NOISE) {
+      if (CENTRED) {
+        // the fast stream: float(p) +- c in one v_fma_mix_f32, then the code off the float
+        const float zl = NEG ? widen_sub_lo(p, u[2 * j]) : widen_add_lo(p, u[2 * j]);
+        const float zh = NEG ? widen_sub_hi(p, u[2 * j + 1]) : widen_add_hi(p, u[2 * j + 1]);
+        c[2 * j] = ANY ? centred_code_bits_of_any(zl) : centred_code_bits_of(zl);
+        c[2 * j + 1] = ANY ? centred_code_bits_of_any(zh) : centred_code_bits_of(zh);
+      } else if (CONST_NOISE) {
         // u = 0.5: float(p) + 0.5 and the following - 0.5 are both exact for every half p (at most 24
         // significant bits between 2^-1 and p's last bit), so y - 0.5 == float(p) and the code is
         // rint(float(p)): float(p) plus the constant rounds to the constant + rint(float(p))
@@ -511,17 +543,18 @@ template <> struct Elem<bf16> {
   __device__ static __forceinline__ float make_scale(float lo, float hi, int qmax) {
     return Elem<float>::make_scale(lo, hi, qmax);
   }
-  template <bool ANY>
+  template <bool ANY, bool CENTRED = false>
   __device__ static __forceinline__ uint32_t code1(const Store& st, int k, int e, float mn, float s, float u) {
     float t = widen(st, k, e) - mn;
     float y = __builtin_fmaf(t, s, u);
+    if (CENTRED) return ANY ? rint_clamp0<true>(y) : centred_code_bits_of(y);
     return ANY ? rint_clamp0<true>(y - 0.5f) : code_bits_of(y);
   }
-  template <bool CONST_NOISE, bool ANY>
+  template <bool CONST_NOISE, bool ANY, bool CENTRED = false, bool NEG = false>
   __device__ static __forceinline__ void codes(const Store& st, int k, float mn, float s, const float (&u)[8],
                                                uint32_t (&c)[8]) {
 #pragma unroll
-    for (int e = 0; e < 8; e++) c[e] = code1<ANY>(st, k, e, mn, s, u[e]);
+    for (int e = 0; e < 8; e++) c[e] = code1<ANY, CENTRED>(st, k, e, mn, s, NEG ? -u[e] : u[e]);
   }
   static constexpr bool kRepairsInfiniteScale = false;
   __device__ static __forceinline__ bool scale_is_inf(float) { return false; }
@@ -579,62 +612,89 @@ template <int LANE> __device__ __forceinline__ f16 row_bcast(f16 v) {
   return __builtin_bit_cast(f16, (uint16_t)row_bcast_u32<LANE>((uint32_t)__builtin_bit_cast(uint16_t, v)));
 }
 
-// 16-bit piece e of a pair of Philox words -> uniform of the fast stream
-__device__ __forceinline__ float fast_piece(uint32_t w0, uint32_t w1, int e) {
-  const uint32_t w = (e & 2) ? w1 : w0;
-  return fast_uniform_map((e & 1) ? (w >> 16) : (w & 0xffffu));
-}
 // swap with the neighbouring lane (lane ^ 1): DPP quad_perm [1,0,3,2]
 __device__ __forceinline__ uint32_t swap_with_neighbour(uint32_t v) {
   return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0xB1, 0xf, 0xf, false);
 }
 
-// The fast stream.  A group of 256 elements draws 16 Philox blocks; block j serves columns 8j .. 8j+7 with its
-// eight 16-bit pieces h (word by word, low half first): u = (h + 0.5) * 2^-16.  The column 128 further on
-// takes 1 - u, the same draw mirrored: every element's noise is uniform on the same grid, and the two elements of
-// a pair (which sit half a group apart) round in opposite directions more often than not (their rounding errors
-// have covariance <= 0).  Half the Philox work, and no second conversion for the mirrored half.
-// In terms of the flat element index E: block (E / 256) * 16 + (E % 128) / 8, piece E % 8, mirrored if E % 256 >= 128.
-__device__ __forceinline__ uint64_t fast_block_of(uint64_t E) { return (E >> 8) * 16 + ((E & 127) >> 3); }
-__device__ __forceinline__ float fast_mirror(float u) { return 1.0f - u; }   // exact: u has 17 significant bits
+// The fast stream.  Two consecutive groups (512 elements) draw 16 Philox blocks; block j serves columns 8j .. 8j+7 of
+// both: its bytes 0..7 (word by word, low byte first) the first group's, bytes 8..15 the second's, one byte h per
+// element, taken as the centred draw c = (2h - 255) / 512.  The column 128 further on takes -c, the same draw
+// mirrored: every element's noise is uniform on the same 256-point grid, symmetric about 0 and strictly inside
+// (-1/2, 1/2), and the two elements of a pair (which sit half a group apart) round in opposite directions more
+// often than not (their rounding errors have covariance <= 0).  One block per 32 elements, one conversion and one
+// fma per two elements (the mirrored draw is a sign flip that folds into the instruction that adds it).
+// In terms of the flat element index E: block (E / 512) * 16 + (E % 128) / 8, byte ((E / 256) % 2) * 8 + E % 8,
+// mirrored if E % 256 >= 128.
+__device__ __forceinline__ uint64_t fast_block_of(uint64_t E) { return (E >> 9) * 16 + ((E & 127) >> 3); }
+// the centred draw of element E from the words of its block
+__device__ __forceinline__ float fast_centred_of(const uint32_t (&r)[4], uint64_t E) {
+  const int b = (int)(((E >> 8) & 1) * 8 + (E & 7));
+  const uint32_t w = (b & 8) ? ((b & 4) ? r[3] : r[2]) : ((b & 4) ? r[1] : r[0]);
+  const float c = fast_centred_map(w, b & 3);
+  return (E & 128) ? -c : c;
+}
 
-// The fast stream's uniforms for all chunks of group n that lane i owns.  With 8-column chunks (8i + 128m) the
-// lane's two chunks are one block and its mirror image.  With 4-column chunks (4i + 64m) chunks 0 and 1 are halves
-// of blocks i/2 and 8 + i/2, which two neighbouring lanes share: the even lane computes the first, the odd lane the
-// second, and they exchange the halves the other one needs; chunks 2 and 3 are the mirror images of 0 and 1.
+// The two words of each group of the pair `pair` that row lane i needs: w[g][0..1] hold the 8 draws of the lane's
+// unmirrored columns of group 2 * pair + g, in column order.  With 8-column chunks (8i + 128m) that is the lane's
+// own block.  With 4-column chunks (4i + 64m) chunks 0 and 1 are halves of blocks i/2 and 8 + i/2, which two
+// neighbouring lanes share: the even lane computes the first, the odd lane the second, and they exchange the words
+// the other one needs (the even lane owns words 0 and 2 of a block, the odd lane words 1 and 3).
 template <typename T>
-__device__ __forceinline__ void fast_noise(int64_t n, int i, uint32_t k0, uint32_t k1,
-                                           float (&u)[Elem<T>::kQChunks][Elem<T>::kQWidth]) {
+__device__ __forceinline__ void fast_pair_words(int64_t pair, int i, uint32_t k0, uint32_t k1, uint32_t (&w)[2][2]) {
   constexpr int CH = Elem<T>::kQChunks, W = Elem<T>::kQWidth;
   uint32_t r[4];
   if (W == 8) {
     static_assert(W != 8 || CH == 2, "two chunks of 8 columns, 128 apart");
-    const uint64_t blk = (uint64_t)n * 16 + i;
+    const uint64_t blk = (uint64_t)pair * 16 + i;
     philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
-#pragma unroll
-    for (int e = 0; e < W; e++) {
-      u[0][e] = fast_piece(r[(e >> 2) * 2], r[(e >> 2) * 2 + 1], e & 3);
-      u[CH - 1][e] = fast_mirror(u[0][e]);
-    }
+    w[0][0] = r[0]; w[0][1] = r[1]; w[1][0] = r[2]; w[1][1] = r[3];
   } else {
     static_assert(W == 8 || CH == 4, "four chunks of 4 columns, 64 apart");
     const bool odd = i & 1;
-    const uint64_t blk = (uint64_t)n * 16 + (odd ? 8 : 0) + (i >> 1);
+    const uint64_t blk = (uint64_t)pair * 16 + (odd ? 8 : 0) + (i >> 1);
     philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
-    // the even lane owns elements 0..3 of a block (words 0,1), the odd lane elements 4..7 (words 2,3)
-    const uint32_t ga = swap_with_neighbour(odd ? r[0] : r[2]);
-    const uint32_t gb = swap_with_neighbour(odd ? r[1] : r[3]);
-    const uint32_t a0 = odd ? ga : r[0], a1 = odd ? gb : r[1];   // chunk 0: block i/2
-    const uint32_t b0 = odd ? r[2] : ga, b1 = odd ? r[3] : gb;   // chunk 1: block 8 + i/2
-#pragma unroll
-    for (int e = 0; e < W; e++) {
-      u[0][e] = fast_piece(a0, a1, e);
-      u[1 % CH][e] = fast_piece(b0, b1, e);
-      u[2 % CH][e] = fast_mirror(u[0][e]);
-      u[3 % CH][e] = fast_mirror(u[1 % CH][e]);
-    }
+    const uint32_t g0 = swap_with_neighbour(odd ? r[0] : r[1]);
+    const uint32_t g1 = swap_with_neighbour(odd ? r[2] : r[3]);
+    w[0][0] = odd ? g0 : r[0];   // chunk 0: block i/2
+    w[0][1] = odd ? r[1] : g0;   // chunk 1: block 8 + i/2
+    w[1][0] = odd ? g1 : r[2];
+    w[1][1] = odd ? r[3] : g1;
   }
 }
+// The centred draws of the lane's unmirrored chunks (the first half of its chunks) from the group's two words: draw
+// k * W + e belongs to element e of chunk k; chunk k + CH/2 takes the same draws negated.
+template <typename T>
+__device__ __forceinline__ void fast_centred_draws(const uint32_t (&w)[2], float (&c)[Elem<T>::kQChunks / 2][Elem<T>::kQWidth]) {
+  constexpr int CH = Elem<T>::kQChunks, W = Elem<T>::kQWidth;
+#pragma unroll
+  for (int k = 0; k < CH / 2; k++)
+#pragma unroll
+    for (int e = 0; e < W; e++) {
+      const int f = k * W + e;
+      c[k][e] = (f & 2) ? ((f & 1) ? fast_centred_map<3>(w[f >> 2]) : fast_centred_map<2>(w[f >> 2]))
+                        : ((f & 1) ? fast_centred_map<1>(w[f >> 2]) : fast_centred_map<0>(w[f >> 2]));
+    }
+}
+// The state of the fast stream along a row's groups: group g of the row (first group n0) draws from the words of its
+// pair, which are computed when the row enters the pair.  Rows of two or more groups start on an even group, so that
+// happens at every even g; a row of one group computes its pair's block and takes its half.
+template <typename T, int GPR>
+struct FastRow {
+  uint32_t w[2][2];
+  __device__ __forceinline__ void draws(int g, int64_t n0, int i, uint32_t k0, uint32_t k1,
+                                        float (&c)[Elem<T>::kQChunks / 2][Elem<T>::kQWidth]) {
+    if (GPR == 1) {
+      const int64_t n = n0 + g;
+      fast_pair_words<T>(n >> 1, i, k0, k1, w);
+      const uint32_t mine[2] = {(n & 1) ? w[1][0] : w[0][0], (n & 1) ? w[1][1] : w[0][1]};
+      fast_centred_draws<T>(mine, c);
+    } else {
+      if ((g & 1) == 0) fast_pair_words<T>((n0 + g) >> 1, i, k0, k1, w);
+      fast_centred_draws<T>(w[g & 1], c);
+    }
+  }
+};
 
 // ------------------------------------------------------------------------------------------------
 // Quantize SGR consecutive super-groups (one 16-lane row): all their groups are loaded first, reduced, and share
@@ -676,6 +736,7 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
         for (int k = 0; k < CH; k++) Elem<T>::load_chunk(x + (n0 + g) * GROUP + chunk_col<T>(k, i), v[g], k);
     }
     uint32_t bytes[CH][W];
+    FastRow<T, GPR> fast;
 #pragma unroll
     for (int g0 = 0; g0 < GPR; g0 += ST) {
       if (LAZY) {
@@ -723,10 +784,19 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
 #pragma unroll
             for (int e = 0; e < W; e++) bytes[k][e] = 0;
         }
-        float u[CH][W];
         if (NOISE == GACT_NOISE_FAST) {
-          fast_noise<T>(n, i, k0, k1, u);
+          float cd[CH / 2][W];
+          fast.draws(g, n0, i, k0, k1, cd);
+#pragma unroll
+          for (int k = 0; k < CH; k++) {
+            uint32_t c[W];
+            if (k < CH / 2) Elem<T>::template codes<false, GIVEN, true, false>(v[g], k, lo_s[j], sc_s[j], cd[k % (CH / 2)], c);
+            else Elem<T>::template codes<false, GIVEN, true, true>(v[g], k, lo_s[j], sc_s[j], cd[k % (CH / 2)], c);
+#pragma unroll
+            for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (ni * BITS);
+          }
         } else {
+          float u[CH][W];
 #pragma unroll
           for (int k = 0; k < CH; k++) {
             if (NOISE == GACT_NOISE_INJECT) {
@@ -736,13 +806,13 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
               for (int e = 0; e < W; e++) u[k][e] = 0.5f;
             }
           }
-        }
 #pragma unroll
-        for (int k = 0; k < CH; k++) {
-          uint32_t c[W];
-          Elem<T>::template codes<NOISE == GACT_NOISE_CONST, GIVEN>(v[g], k, lo_s[j], sc_s[j], u[k], c);
+          for (int k = 0; k < CH; k++) {
+            uint32_t c[W];
+            Elem<T>::template codes<NOISE == GACT_NOISE_CONST, GIVEN>(v[g], k, lo_s[j], sc_s[j], u[k], c);
 #pragma unroll
-          for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (ni * BITS);
+            for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (ni * BITS);
+          }
         }
         if (Elem<T>::kRepairsInfiniteScale && __builtin_amdgcn_ballot_w64(Elem<T>::scale_is_inf(sc_s[j])) != 0) {
           if (Elem<T>::scale_is_inf(sc_s[j])) {
@@ -818,6 +888,7 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
     }
   }
 
+  FastRow<T, GPR> fast;
 #pragma unroll
   for (int q = 0; q < SGR; q++) {
     const int64_t sg = sg0 + q;
@@ -852,10 +923,19 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
         const int g = q * WPT + ni;
         const int64_t n = n0 + g;
         if (n < N) {
-          float u[CH][W];
           if (NOISE == GACT_NOISE_FAST) {
-            fast_noise<T>(n, i, k0, k1, u);
+            float cd[CH / 2][W];
+            fast.draws(g, n0, i, k0, k1, cd);
+#pragma unroll
+            for (int k = 0; k < CH; k++) {
+              uint32_t c[W];
+              if (k < CH / 2) Elem<T>::template codes<false, GIVEN, true, false>(v[g], k, lo_t[g], s_t[g], cd[k % (CH / 2)], c);
+              else Elem<T>::template codes<false, GIVEN, true, true>(v[g], k, lo_t[g], s_t[g], cd[k % (CH / 2)], c);
+#pragma unroll
+              for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (ni * BITS);
+            }
           } else {
+            float u[CH][W];
 #pragma unroll
             for (int k = 0; k < CH; k++) {
               if (NOISE == GACT_NOISE_INJECT) {
@@ -865,13 +945,13 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
                 for (int e = 0; e < W; e++) u[k][e] = 0.5f;
               }
             }
-          }
 #pragma unroll
-          for (int k = 0; k < CH; k++) {
-            uint32_t c[W];
-            Elem<T>::template codes<NOISE == GACT_NOISE_CONST, GIVEN>(v[g], k, lo_t[g], s_t[g], u[k], c);
+            for (int k = 0; k < CH; k++) {
+              uint32_t c[W];
+              Elem<T>::template codes<NOISE == GACT_NOISE_CONST, GIVEN>(v[g], k, lo_t[g], s_t[g], u[k], c);
 #pragma unroll
-            for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (ni * BITS);
+              for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << (ni * BITS);
+            }
           }
         }
       }
@@ -1391,13 +1471,11 @@ pack_any_kernel(const T* __restrict__ data, const T* __restrict__ mn, const T* _
     } else if (NOISE == GACT_NOISE_FAST) {
       const uint64_t blk = fast_block_of((uint64_t)id);
       philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r);
-      const int e = (int)(id & 7);
-      u = fast_uniform_map((e & 1) ? (r[e >> 1] >> 16) : (r[e >> 1] & 0xffffu));
-      if (id & 128) u = fast_mirror(u);
+      u = fast_centred_of(r, (uint64_t)id);
     }
     typename Elem<T>::Store one;
     Elem<T>::set(one, 0, 0, data[id]);
-    byte |= Elem<T>::template code1<true>(one, 0, 0, mn[sid], scale[sid], u) << (ni * bits);
+    byte |= Elem<T>::template code1<true, NOISE == GACT_NOISE_FAST>(one, 0, 0, mn[sid], scale[sid], u) << (ni * bits);
   }
   packed[j] = (uint8_t)byte;
 }
@@ -1459,13 +1537,11 @@ pack_rows8_kernel(const T* __restrict__ data, const T* __restrict__ mn, const T*
         u[e] = curand_uniform_map(r[e][ni & 3]);
       }
     } else if (NOISE == GACT_NOISE_FAST) {
+      // the thread's 8 consecutive elements share a block (id0 is a multiple of 8)
       const uint64_t blk = fast_block_of((uint64_t)id0);
       philox4x32<PHILOX_FAST_ROUNDS>(0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32), k0, k1, r[0]);
 #pragma unroll
-      for (int e = 0; e < 8; e++) {
-        u[e] = fast_uniform_map((e & 1) ? (r[0][e >> 1] >> 16) : (r[0][e >> 1] & 0xffffu));
-        if (id0 & 128) u[e] = fast_mirror(u[e]);
-      }
+      for (int e = 0; e < 8; e++) u[e] = fast_centred_of(r[0], (uint64_t)id0 + e);
     } else {
 #pragma unroll
       for (int e = 0; e < 8; e++) u[e] = 0.5f;
@@ -1474,7 +1550,7 @@ pack_rows8_kernel(const T* __restrict__ data, const T* __restrict__ mn, const T*
     for (int e = 0; e < 8; e++) {
       typename Elem<T>::Store one;
       Elem<T>::set(one, 0, 0, x[e]);
-      bytes[e] |= Elem<T>::template code1<true>(one, 0, 0, lo, sc, u[e]) << (ni * bits);
+      bytes[e] |= Elem<T>::template code1<true, NOISE == GACT_NOISE_FAST>(one, 0, 0, lo, sc, u[e]) << (ni * bits);
     }
   }
   u32x2 w;

@@ -46,8 +46,12 @@ class QuantizationConfig:
         self.device_seed = False
 
         # ---- stochastic-rounding noise (not in the reference) ----
-        # "fast":          one Philox4x32-7 block per 16 elements (8 draws of 16 bits, each used once as u and once,
-        #                  half a group further on, as 1 - u)
+        # "fast":          one Philox4x32-7 block per 32 elements: 16 draws of 8 bits, centred ((2h - 255)/512, so the
+        #                  reference's "+ noise - 0.5" is one addition), each used once as c and once, half a group
+        #                  further on, as -c.  The two elements of such a pair are not independent: their rounding
+        #                  errors have covariance <= 0, which lowers the variance of a sum in which both carry
+        #                  weights of the same sign and raises it (at most twofold) where the signs differ; over
+        #                  weights of random sign it equals the independent stream's.
         # "reference":     the reference's stream (one Philox state per output byte, cuRAND uniform map)
         # "deterministic": u = 0.5 everywhere, i.e. round to nearest
         self.rng_stream = "fast"

@@ -33,7 +33,7 @@ extern "C" {
 #define GACT_NOISE_INJECT 1 /* u read from a float tensor laid out like the (padded) data        */
 #define GACT_NOISE_REF 2    /* the reference's stream: one Philox4x32-10 state per output byte,  */
                             /* (seed, subsequence = byte index, offset 0), cuRAND uniform map    */
-#define GACT_NOISE_FAST 3   /* one Philox4x32-7 block per 8 consecutive elements, 16-bit noise   */
+#define GACT_NOISE_FAST 3   /* one Philox4x32-7 block per 32 elements, 8-bit centred noise (ours)  */
 
 #define GACT_OK 0
 #define GACT_EINVAL (-1) /* bad argument (bits not in {1,2,4,8}, negative size, null pointer ...) */

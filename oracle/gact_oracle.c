@@ -246,35 +246,43 @@ static inline float ref_stream_uniform(uint64_t seed, uint64_t byte_index, int d
 /* The fast noise stream (ours; the reference has no counterpart).  Philox4x32 */
 /* with seven rounds (the same round function; the fewest rounds for which    */
 /* Random123's authors report that the generator passes BigCrush; its         */
-/* kat_vectors hold the 7-round known answers too), key = seed.  Every 256    */
-/* consecutive elements of the flattened tensor draw 16 blocks: element E     */
-/* takes block (E/256)*16 + (E%128)/8 (counter = (0, 0, block lo, block hi)),  */
-/* of it the 16-bit piece E%8 (word (E%8)/2, low half first), h;               */
-/* u = (h + 0.5) * 2^-16 for E%256 < 128 and 1 - that for E%256 >= 128: the    */
-/* two elements half a group apart share one draw, mirrored (an antithetic     */
-/* pair: both uniform on the same grid, strictly inside (0, 1), symmetric      */
-/* about 1/2; covariance of their rounding errors <= 0).                       */
+/* kat_vectors hold the 7-round known answers too), key = seed.  Every 512    */
+/* consecutive elements of the flattened tensor (two groups of 256) draw 16   */
+/* blocks of 16 bytes.  Element E, with column d = E%256 and d' = d%128:      */
+/* block (E/512)*16 + d'/8 (counter = (0, 0, block lo, block hi)), of its 16  */
+/* output bytes (word by word, low byte first) byte ((E/256)%2)*8 + d'%8, h.   */
+/* The draw is centred: c = (2h - 255)/512, i.e. (h + 0.5)/256 - 1/2, one of  */
+/* 256 values symmetric about 0, strictly inside (-1/2, 1/2); for d >= 128    */
+/* the element takes -c: the two elements half a group apart share one draw,  */
+/* mirrored (an antithetic pair: both uniform on the same grid; covariance of */
+/* their rounding errors <= 0).  The code is rint(max(y, 0)) with the noise   */
+/* added where the reference adds its own: y = fma(x - min, scale, c) for      */
+/* float, float(half product) + c for half - the reference's                   */
+/* (.. + u) - 0.5 with u = c + 1/2, rounded once instead of twice.             */
 #define GACT_FAST_ROUNDS 7
-static inline float fast_stream_uniform_from_block(const uint32_t out[4], int e8) {
-  uint32_t w = out[e8 >> 1];
-  uint32_t h = (e8 & 1) ? (w >> 16) : (w & 0xffffu);
-  return (float)(2u * h + 1u) * 7.62939453125e-06f; /* (2h+1) * 2^-17, exact */
+static inline uint64_t fast_stream_block(uint64_t elem) { return (elem >> 9) * 16u + ((elem & 127u) >> 3); }
+static inline int fast_stream_byte(uint64_t elem) { return (int)(((elem >> 8) & 1u) * 8u + (elem & 7u)); }
+static inline float fast_stream_centred_from_block(const uint32_t out[4], uint64_t elem) {
+  int b = fast_stream_byte(elem);
+  uint32_t h = (out[b >> 2] >> (8 * (b & 3))) & 0xffu;
+  float c = (float)(2 * (int32_t)h - 255) * 0.001953125f; /* (2h - 255) * 2^-9, exact */
+  return (elem & 128u) ? -c : c;
 }
-static inline uint64_t fast_stream_block(uint64_t elem) { return (elem >> 8) * 16u + ((elem & 127u) >> 3); }
-static inline float fast_stream_uniform(uint64_t seed, uint64_t elem) {
+static inline float fast_stream_centred(uint64_t seed, uint64_t elem) {
   uint64_t blk = fast_stream_block(elem);
   uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
   uint32_t ctr[4] = {0u, 0u, (uint32_t)blk, (uint32_t)(blk >> 32)};
   uint32_t out[4];
   gact_oracle_philox4x32(ctr, key, GACT_FAST_ROUNDS, out);
-  float u = fast_stream_uniform_from_block(out, (int)(elem & 7));
-  return (elem & 128u) ? 1.0f - u : u; /* exact: 17 significant bits */
+  return fast_stream_centred_from_block(out, elem);
 }
+/* the same draw as a uniform on (0, 1): c + 1/2 = (2h + 1)/512, exact */
+static inline float fast_stream_uniform(uint64_t seed, uint64_t elem) { return fast_stream_centred(seed, elem) + 0.5f; }
 
 #define GACT_NOISE_CONST 0  /* u = 0.5 for every element: deterministic rounding */
 #define GACT_NOISE_INJECT 1 /* u read from a float tensor shaped like the data  */
 #define GACT_NOISE_REF 2    /* the reference's cuRAND-compatible stream         */
-#define GACT_NOISE_FAST 3   /* one 7-round Philox block per 8 elements, 16-bit noise */
+#define GACT_NOISE_FAST 3   /* one 7-round Philox block per 32 elements, 8-bit centred noise */
 
 /* Materialise the noise tensor a given mode uses, in data layout [N,G,D].    */
 void gact_oracle_noise(int noise_mode, uint64_t seed, int bits, int64_t N, int64_t G, int64_t D, float* u) {
@@ -335,6 +343,21 @@ static inline int32_t code_f16(uint16_t x, uint16_t mn, uint16_t s, float u) {
   z = (z > 0.0f) ? z : 0.0f;
   return float2int_rn_sat(z);
 }
+/* The fast stream's form of the same code: the draw c is centred, so the      */
+/* reference's "+ noise - 0.5" is one addition.                                 */
+static inline int32_t code_f32_centred(float x, float mn, float s, float c) {
+  float t = x - mn;
+  float z = fmaf(t, s, c);
+  z = (z > 0.0f) ? z : 0.0f;
+  return float2int_rn_sat(z);
+}
+static inline int32_t code_f16_centred(uint16_t x, uint16_t mn, uint16_t s, float c) {
+  float t = rh(h2f(x) - h2f(mn));
+  float p = rh(t * h2f(s));
+  float z = p + c;
+  z = (z > 0.0f) ? z : 0.0f;
+  return float2int_rn_sat(z);
+}
 
 /* P3/P4  pack.  quantization_cuda_kernel.cu:38-71 (kernel) and :74-146       */
 /* (launcher).  Output byte j = (no*G + g)*D + d ORs, for ni < 8/bits with    */
@@ -351,7 +374,6 @@ void gact_oracle_pack(const void* data, const void* mn, const void* scale, int d
   for (int64_t no = 0; no < n_outer; no++) {
     for (int64_t g = 0; g < G; g++) {
       for (int64_t d0 = 0; d0 < D; d0 += 8) {
-        /* 8 columns at a time so that the fast stream computes each block once */
         for (int64_t d = d0; d < d0 + 8 && d < D; d++) {
           int64_t j = (no * G + g) * D + d;
           uint8_t byte = 0;
@@ -360,13 +382,18 @@ void gact_oracle_pack(const void* data, const void* mn, const void* scale, int d
             if (n >= N) break;
             int64_t id = (n * G + g) * D + d;
             int64_t sid = n * G + g;
-            float u;
-            if (noise_mode == GACT_NOISE_CONST) u = 0.5f;
-            else if (noise_mode == GACT_NOISE_INJECT) u = noise[id];
+            float u = 0.5f;
+            if (noise_mode == GACT_NOISE_INJECT) u = noise[id];
             else if (noise_mode == GACT_NOISE_REF) u = ref_stream_uniform(seed, (uint64_t)j, ni);
-            else u = fast_stream_uniform(seed, (uint64_t)id);
+            else if (noise_mode == GACT_NOISE_FAST) u = fast_stream_centred(seed, (uint64_t)id);
             int32_t val;
-            if (dtype == GACT_F32)
+            if (noise_mode == GACT_NOISE_FAST) {
+              if (dtype == GACT_F32)
+                val = code_f32_centred(((const float*)data)[id], ((const float*)mn)[sid], ((const float*)scale)[sid], u);
+              else
+                val = code_f16_centred(((const uint16_t*)data)[id], ((const uint16_t*)mn)[sid],
+                                       ((const uint16_t*)scale)[sid], u);
+            } else if (dtype == GACT_F32)
               val = code_f32(((const float*)data)[id], ((const float*)mn)[sid], ((const float*)scale)[sid], u);
             else
               val = code_f16(((const uint16_t*)data)[id], ((const uint16_t*)mn)[sid],

@@ -246,19 +246,21 @@ def test_more_than_2_to_31_elements(bits):
     Nt = (tail.size + 255) // 256
     # the oracle numbers elements from 0, so feed it the absolute indices through an injected noise tensor
     idx = (np.arange(Nt * 256, dtype=np.uint64) + np.uint64(g0 * 256))
-    # element E draws block (E/256)*16 + (E%128)/8, piece E%8, mirrored in the upper half of every 256
-    blk = (idx >> np.uint64(8)) * np.uint64(16) + ((idx & np.uint64(127)) >> np.uint64(3))
+    # element E draws block (E/512)*16 + (E%128)/8, byte ((E/256)%2)*8 + E%8, c = (2h - 255)/512, negated in the
+    # upper half of every 256; injected as the uniform c + 1/2 (for half data the reference form's two additions
+    # are exact, so it gives the same codes)
+    blk = (idx >> np.uint64(9)) * np.uint64(16) + ((idx & np.uint64(127)) >> np.uint64(3))
     uu = np.empty(Nt * 256, np.float32)
     cache = {}
     for b in np.unique(blk[:512]):                      # the blocks of the first two groups are enough to pin the indexing
         cache[int(b)] = oracle.philox4x32([0, 0, int(b) & 0xFFFFFFFF, int(b) >> 32], [9, 0], oracle.FAST_ROUNDS)
     sel = np.arange(512)
     for e in sel:
-        w = int(cache[int(blk[e])][(int(idx[e]) % 8) // 2])
-        h = (w >> 16) if (int(idx[e]) % 2) else (w & 0xFFFF)
-        uu[e] = (h + 0.5) / 65536.0
-        if int(idx[e]) % 256 >= 128:
-            uu[e] = np.float32(1.0) - uu[e]
+        E = int(idx[e])
+        byte = ((E // 256) % 2) * 8 + E % 8
+        h = (int(cache[int(blk[e])][byte // 4]) >> (8 * (byte % 4))) & 0xFF
+        c = (2 * h - 255) / 512.0
+        uu[e] = (-c if E % 256 >= 128 else c) + 0.5
     first = int(sel.max()) + 1                          # the selected elements are the first 512 of the tail
     assert first == 512
     ref = oracle.op_quantize(tail[:512], bits, oracle.NOISE_INJECT, 0, uu[:512])

@@ -150,27 +150,64 @@ def test_reference_stream_walks_the_counter_like_curand():
 
 
 def fast_stream_expected(seed, E):
-    """The fast stream restated from its definition: block (E/256)*16 + (E%128)/8 of Philox4x32-7, piece E%8,
-    u = (h + 0.5) / 2^16, mirrored (1 - u) in the upper half of every 256."""
-    blk = (E // 256) * 16 + (E % 128) // 8
+    """The fast stream restated from its definition: block (E/512)*16 + (E%128)/8 of Philox4x32-7, of its 16 bytes
+    byte ((E/256)%2)*8 + E%8, c = (2h - 255)/512, negated in the upper half of every 256; as a uniform: c + 1/2."""
+    blk = (E // 512) * 16 + (E % 128) // 8
     out = oracle.philox4x32([0, 0, blk & 0xFFFFFFFF, blk >> 32], [seed & 0xFFFFFFFF, seed >> 32], oracle.FAST_ROUNDS)
-    w = int(out[(E % 8) // 2])
-    h = (w >> 16) if (E % 2) else (w & 0xFFFF)
-    u = Fraction(2 * h + 1, 1 << 17)
-    return float(1 - u if E % 256 >= 128 else u)
+    b = ((E // 256) % 2) * 8 + E % 8
+    h = (int(out[b // 4]) >> (8 * (b % 4))) & 0xFF
+    c = Fraction(2 * h - 255, 512)
+    return float((-c if E % 256 >= 128 else c) + Fraction(1, 2))
 
 
 def test_fast_stream_definition():
     seed = 7
-    u = oracle.noise(oracle.NOISE_FAST, seed, 4, 3).reshape(-1)
-    for E in (0, 1, 7, 8, 127, 128, 129, 135, 255, 256, 300, 383, 384, 500, 767):
+    u = oracle.noise(oracle.NOISE_FAST, seed, 4, 5).reshape(-1)
+    for E in (0, 1, 7, 8, 127, 128, 129, 135, 255, 256, 263, 300, 383, 384, 500, 511, 512, 767, 768, 1023, 1279):
         assert u[E] == np.float32(fast_stream_expected(seed, E)), E
     assert 0.0 < u.min() and u.max() < 1.0
-    # the two halves of every 256 are mirror images, and every value sits on the (k + 0.5) / 2^16 grid
-    g = u.reshape(3, 2, 128)
+    # the two halves of every 256 are mirror images, and every value sits on the (k + 0.5) / 256 grid
+    g = u[:1024].reshape(4, 2, 128)
     assert np.array_equal(g[:, 1, :], np.float32(1.0) - g[:, 0, :])
-    k = u.astype(np.float64) * 65536.0 - 0.5
-    assert np.array_equal(k, np.round(k)) and k.min() >= 0 and k.max() <= 65535
+    k = u.astype(np.float64) * 256.0 - 0.5
+    assert np.array_equal(k, np.round(k)) and k.min() >= 0 and k.max() <= 255
+    # all 16 bytes of a block are used, each once: 32 elements per block
+    seen = {}
+    for E in range(512):
+        blk = (E // 512) * 16 + (E % 128) // 8
+        seen.setdefault(blk, []).append((((E // 256) % 2) * 8 + E % 8, E % 256 >= 128))
+    assert sorted(seen) == list(range(16))
+    assert all(sorted(v) == sorted((b, m) for b in range(16) for m in (False, True)) for v in seen.values())
+
+
+def test_fast_stream_code_is_the_reference_code_with_one_rounding():
+    """The fast stream's code is rint(max(z, 0)) with z = (x - min) * scale + c (float: one fma; half: the half
+    product widened, + c), c the centred draw: the reference's rint(max((.. + u) - 0.5, 0)) with u = c + 1/2 and
+    the two additions merged.  Checked against exact rational arithmetic on the oracle's own scale and min, and
+    against the reference form under the same noise injected (they may only differ where the reference's
+    first rounding moved a sum across a tie)."""
+    rng = np.random.default_rng(12)
+    for dtype in (np.float32, np.float16):
+        for bits in (1, 2, 4, 8):
+            x = (rng.standard_normal((6, 256)) * 3).astype(dtype)
+            q = oracle.op_quantize(x, bits, oracle.NOISE_FAST, 21)
+            codes = unpack_codes(q[0], bits, 6)
+            u = oracle.noise(oracle.NOISE_FAST, 21, bits, 6).reshape(6, 256)
+            mn, sc = q[3].reshape(-1), q[2].reshape(-1)
+            for n in range(6):
+                for d in range(0, 256, 5):
+                    c = F(u[n, d]) - Fraction(1, 2)
+                    if dtype == np.float32:
+                        t = round_fraction(F(x[n, d]) - F(mn[n]), np.float32)
+                        z = round_fraction(F(t) * F(sc[n]) + c, np.float32)          # one rounding: fused multiply-add
+                    else:
+                        t = round_fraction(F(x[n, d]) - F(mn[n]), np.float16)
+                        prod = round_fraction(F(t) * F(sc[n]), np.float16)
+                        z = round_fraction(F(prod) + c, np.float32)
+                    want = rne_int(F(z)) if z > 0 else 0
+                    assert codes[n, d] == want & (2 ** bits - 1), (dtype, bits, n, d)
+            same = oracle.op_quantize(x, bits, oracle.NOISE_INJECT, 0, u)
+            assert (unpack_codes(same[0], bits, 6) != codes).mean() < 1e-3
 
 
 def test_fast_stream_marginals_and_pair_covariance():
@@ -180,6 +217,9 @@ def test_fast_stream_marginals_and_pair_covariance():
     assert abs(u.mean() - 0.5) < 2e-3 and abs(u.var() - 1.0 / 12.0) < 2e-3
     lower, upper = u[:, :128], u[:, 128:]
     assert abs(lower.mean() - 0.5) < 2e-3 and abs(upper.mean() - 0.5) < 2e-3
+    # every one of the 256 grid points is drawn equally often
+    hist = np.bincount(np.round(lower * 256 - 0.5).astype(int).reshape(-1), minlength=256)
+    assert hist.min() > 0.9 * lower.size / 256 and hist.max() < 1.1 * lower.size / 256
     for fi, fj in ((0.3, 0.3), (0.7, 0.6), (0.5, 0.5), (0.9, 0.2)):
         up_i = lower >= 1.0 - fi
         up_j = upper >= 1.0 - fj
@@ -187,9 +227,43 @@ def test_fast_stream_marginals_and_pair_covariance():
         cov = (up_i & up_j).mean() - up_i.mean() * up_j.mean()
         want = max(0.0, fi + fj - 1.0) - fi * fj
         assert abs(cov - want) < 5e-3 and cov < 1e-3
-    # neighbours inside a block, and elements of different blocks, are uncorrelated
-    for a, b in ((u[:, 0], u[:, 1]), (u[:, 5], u[:, 77]), (u[:-1, 9], u[1:, 9])):
+    # neighbours inside a block, the two groups that share a block, and elements of different blocks are uncorrelated
+    for a, b in ((u[:, 0], u[:, 1]), (u[:, 5], u[:, 77]), (u[:-1, 9], u[1:, 9]), (u[0::2, 9], u[1::2, 9]),
+                 (u[0::2, 130], u[1::2, 3])):
         assert abs(np.corrcoef(a, b)[0, 1]) < 0.05
+
+
+def test_fast_stream_pairs_in_a_weighted_sum():
+    """A gradient is a weighted sum of rounding errors.  The mirrored pairs are not independent: where the two
+    weights of a pair have the same sign the pair's variance is below the independent stream's, where they
+    have opposite signs above it (at most twice); over weights of random sign the sum's variance equals the
+    independent one's, sum w_i^2 f_i (1 - f_i), which is what AutoPrecision's variance model assumes."""
+    rng = np.random.default_rng(3)
+    groups = 20000
+    u = oracle.noise(oracle.NOISE_FAST, 5, 8, groups).reshape(groups, 256).astype(np.float64)
+    f = rng.random(256)
+    err = (u >= 1.0 - f).astype(np.float64) - f           # rounding error of every element, in code steps
+    independent = (f * (1 - f))
+    for kind in ("random sign", "same sign", "opposite sign"):
+        w = rng.standard_normal(256)
+        if kind == "same sign":
+            w = np.abs(w)
+        elif kind == "opposite sign":
+            w = np.abs(w) * np.where(np.arange(256) < 128, 1.0, -1.0)
+        got = (err @ w).var()
+        model = (w ** 2 * independent).sum()
+        pairs = 2 * (w[:128] * w[128:] * (np.maximum(0.0, f[:128] + f[128:] - 1.0) - f[:128] * f[128:])).sum()
+        assert abs(got / (model + pairs) - 1) < 0.05, kind           # the exact variance with the pair covariances
+        if kind == "same sign":
+            assert got < model
+        elif kind == "opposite sign":
+            assert model < got < 2 * model
+    # averaged over random signs the cross terms vanish
+    ratios = []
+    for trial in range(40):
+        w = rng.standard_normal(256)
+        ratios.append((err[:4000] @ w).var() / (w ** 2 * independent).sum())
+    assert abs(np.mean(ratios) - 1) < 0.05
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
