@@ -720,7 +720,11 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
   typename Elem<T>::Store v[GPR];
   typedef typename Elem<T>::Stat Stat;
   Stat lo_t[GPR], hi_t[GPR], s_t[GPR];
-  if (STAGE > 0 && STAGE < GPR && !GIVEN && NOISE != GACT_NOISE_REF && (n0 + GPR) * GROUP <= numel) {
+  // The staged path is for rows of whole groups.  The choice is made for the wave, not for the row: a wave in which
+  // one row is ragged (the tensor's last) would otherwise run both paths one after the other, each with its own
+  // round trip to memory - and being the tensor's last wave it would hold up the end of the kernel.
+  const bool whole_row = (n0 + GPR) * GROUP <= numel;
+  if (STAGE > 0 && STAGE < GPR && !GIVEN && NOISE != GACT_NOISE_REF && __builtin_amdgcn_ballot_w64(!whole_row) == 0) {
     // All groups whole: the loads in one straight line, then STAGE groups at a time as they arrive: reduce, divide
     // (lane j for group j % STAGE of the stage), encode; a super-group goes out when its last group is done.  The
     // work on the first groups overlaps the loads of the later ones within the wave, which pays where few waves
@@ -1351,11 +1355,136 @@ quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __re
   constexpr int STAGE = SMALL ? G.stage_small : G.stage;
   constexpr bool LAZY = SMALL ? G.lazy_small : G.lazy;
   constexpr int SGR = NOISE == GACT_NOISE_REF ? 1 : G.sgr;   // the reference stream's code is too long to lay out several times
-  const int64_t sg0 = ((int64_t)xcd_tile<(uint32_t)G.run>(blockIdx.x, gridDim.x) * (blockDim.x >> 4) + (threadIdx.x >> 4)) * SGR;
+  // Tiles are handed out last first: the tensor's last tile - the only one that can be ragged, and then slower than
+  // the others (169 343 float groups at 1 bit: 33.4 us when it is dispatched last, 31.6 when first) - goes to the
+  // first workgroup instead of being the one the end of the kernel waits for.
+  const uint32_t tile = gridDim.x - 1u - xcd_tile<(uint32_t)G.run>(blockIdx.x, gridDim.x);
+  const int64_t sg0 = ((int64_t)tile * (blockDim.x >> 4) + (threadIdx.x >> 4)) * SGR;
   if (sg0 * (8 / BITS) >= N) return;
   const uint64_t seed = seed_arg.value();
   quantize_supergroup<T, BITS, NOISE, GIVEN, SGR, STAGE, LAZY>(x, numel, N, sg0, threadIdx.x & 15, packed, scale_out, mn_io, mx_io,
                                                   (uint32_t)seed, (uint32_t)(seed >> 32), noise);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Quantize at 1 bit with a wave per super-group: row r takes groups 2r and 2r + 1 of the 8 whose codes share bytes, the
+// four rows OR their partial bytes together (two ds_bpermute steps on 4 dwords) and each then stores its quarter of the
+// super-group's 256 bytes.  A wave holds 8 KB (float) or 4 KB (half) where a row per super-group makes it hold 32 or
+// 16 KB: on small tensors, where a kernel is mostly its first and last waves, that is 5-15 % (float 2 M elements
+// 5.3 -> 4.8 us, 8 M 9.5 -> 8.3, 13 M 11.5 -> 10.9; half 2 M 5.1 -> 4.7, 4 M 5.4 -> 4.6); from 16 M elements on the two
+// forms are within 2 % of each other (17 M: 13.0 / 13.6, 43 M: 31.4 / 30.6, 103 M: 67.9 / 68.2 us), at 2 bit (two rows
+// per super-group) there is nothing in it at any size.  Same results as quantize_kernel; not for the reference stream.
+// ------------------------------------------------------------------------------------------------
+#ifndef GACT_W8_RUN
+#define GACT_W8_RUN 32
+#endif
+__device__ __forceinline__ uint32_t pack4(const uint32_t* b) {
+  // the reference accumulates in a uint8_t: keep the low 8 bits of every byte
+  return (b[0] & 0xffu) | ((b[1] & 0xffu) << 8) | ((b[2] & 0xffu) << 16) | (b[3] << 24);
+}
+template <typename T, int NOISE>
+__global__ void __launch_bounds__(256)
+quantize_wave8_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
+                      typename Elem<T>::Stat* __restrict__ scale_out, T* __restrict__ mn_out, T* __restrict__ mx_out,
+                      SeedArg seed_arg, const float* __restrict__ noise) {
+  static_assert(NOISE != GACT_NOISE_REF, "the reference stream draws per output byte");
+  typedef typename Elem<T>::Stat Stat;
+  constexpr int BITS = 1, WPT = 8, QMAX = 1;
+  constexpr int CH = Elem<T>::kQChunks, W = Elem<T>::kQWidth;
+  const uint32_t tile = gridDim.x - 1u - xcd_tile<GACT_W8_RUN>(blockIdx.x, gridDim.x);   // last tile first, see quantize_kernel
+  const int64_t sg = (int64_t)tile * (blockDim.x >> 6) + (threadIdx.x >> 6);               // the wave's super-group
+  const int64_t n0 = sg * WPT;
+  if (n0 >= N) return;   // the whole wave
+  const int lane = threadIdx.x & 63, r = lane >> 4, i = lane & 15;
+  const int64_t na = n0 + 2 * r;   // the row's groups: na, na + 1
+  const uint64_t seed = seed_arg.value();
+  const uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+
+  typename Elem<T>::Store v[2];
+#pragma unroll
+  for (int g = 0; g < 2; g++)
+    if (na + g < N) load_group<T>(x, numel, na + g, i, v[g]);
+  Stat lo[2], hi[2], sc[2];
+#pragma unroll
+  for (int g = 0; g < 2; g++) {
+    lo[g] = hi[g] = (Stat)0.0f;
+    if (na + g < N) Elem<T>::group_minmax(v[g], lo[g], hi[g]);
+  }
+  {
+    const bool second = i & 1;   // odd lanes divide for the row's second group
+    const Stat lo_m = second ? lo[1] : lo[0], hi_m = second ? hi[1] : hi[0];
+    const Stat s_m = Elem<T>::make_scale(lo_m, hi_m, QMAX);
+    if (i < 2 && na + i < N) {
+      scale_out[na + i] = s_m;
+      mn_out[na + i] = Elem<T>::elem_of(lo_m);
+      if (mx_out) mx_out[na + i] = Elem<T>::elem_of(hi_m);
+    }
+    sc[0] = row_bcast<0>(s_m);
+    sc[1] = row_bcast<1>(s_m);
+  }
+
+  uint32_t bytes[CH][W];
+#pragma unroll
+  for (int k = 0; k < CH; k++)
+#pragma unroll
+    for (int e = 0; e < W; e++) bytes[k][e] = 0;
+  FastRow<T, 2> fast;
+#pragma unroll
+  for (int g = 0; g < 2; g++) {
+    const int64_t n = na + g;
+    const uint32_t shift = (uint32_t)((2 * r + g) * BITS);   // the group's field within its bytes
+    if (n < N) {
+      if (NOISE == GACT_NOISE_FAST) {
+        float cd[CH / 2][W];
+        fast.draws(g, na, i, k0, k1, cd);
+#pragma unroll
+        for (int k = 0; k < CH; k++) {
+          uint32_t c[W];
+          if (k < CH / 2) Elem<T>::template codes<false, false, true, false>(v[g], k, lo[g], sc[g], cd[k % (CH / 2)], c);
+          else Elem<T>::template codes<false, false, true, true>(v[g], k, lo[g], sc[g], cd[k % (CH / 2)], c);
+#pragma unroll
+          for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << shift;
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < CH; k++) {
+          float u[W];
+          if (NOISE == GACT_NOISE_INJECT) {
+            Elem<T>::load_noise(noise + n * GROUP + chunk_col<T>(k, i), u);
+          } else {
+#pragma unroll
+            for (int e = 0; e < W; e++) u[e] = 0.5f;
+          }
+          uint32_t c[W];
+          Elem<T>::template codes<NOISE == GACT_NOISE_CONST, false>(v[g], k, lo[g], sc[g], u, c);
+#pragma unroll
+          for (int e = 0; e < W; e++) bytes[k][e] |= c[e] << shift;
+        }
+      }
+      if (Elem<T>::kRepairsInfiniteScale && Elem<T>::scale_is_inf(sc[g])) {   // rare, see Elem<T>::kRepairsInfiniteScale
+#pragma unroll
+        for (int k = 0; k < CH; k++)
+#pragma unroll
+          for (int e = 0; e < W; e++)
+            if (Elem<T>::above(v[g], k, e, lo[g])) bytes[k][e] |= 0xffffffffu << shift;
+      }
+    }
+  }
+
+  // the lane's 16 bytes as 4 dwords in the order of their addresses, OR-ed over the four rows (every lane of the wave
+  // is here: only whole waves left above)
+  uint32_t pk[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    pk[j] = pack4(&bytes[j * 4 / W][(j * 4) % W]);
+    pk[j] |= (uint32_t)__shfl_xor((int)pk[j], 16, 64);
+    pk[j] |= (uint32_t)__shfl_xor((int)pk[j], 32, 64);
+  }
+  // row r stores dword r of every lane: float chunk r; half chunk r / 2, its columns 4 (r % 2) .. - 256 contiguous
+  // bytes per store instruction either way
+  const uint32_t mine = r == 0 ? pk[0] : r == 1 ? pk[1] : r == 2 ? pk[2] : pk[3];
+  const int col = W == 4 ? chunk_col<T>(r, i) : chunk_col<T>(r >> 1, i) + 4 * (r & 1);
+  stream_store(mine, reinterpret_cast<uint32_t*>(packed + sg * GROUP + col));
 }
 
 template <typename T, int BITS, bool LARGE = false>
@@ -2185,6 +2314,17 @@ inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
   return 0u;
 }
 
+// Below how many groups a 1-bit quantize takes the wave-per-super-group kernel (0: never), by element size.
+#ifndef GACT_W8_BELOW_F32
+#define GACT_W8_BELOW_F32 57344
+#endif
+#ifndef GACT_W8_BELOW_F16
+#define GACT_W8_BELOW_F16 49152
+#endif
+#ifndef GACT_W8_THREADS
+#define GACT_W8_THREADS 256
+#endif
+
 // the kernel of a noise mode; its small-tensor form where the geometry has one (staging is for fused min/max and
 // not for the reference stream)
 template <typename T, int BITS, int NOISE, bool GIVEN>
@@ -2209,6 +2349,26 @@ int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, typen
                     SeedArg seed, const float* noise, hipStream_t stream) {
   dim3 grid, block;
   constexpr QGeom G = q_geom<T>(BITS);
+  if constexpr (!GIVEN && BITS == 1) {
+    if (noise_mode != GACT_NOISE_REF && N < (sizeof(T) == 4 ? GACT_W8_BELOW_F32 : GACT_W8_BELOW_F16)) {
+      const unsigned per_block = GACT_W8_THREADS / 64;
+      const dim3 wgrid((unsigned)(((N + 7) / 8 + per_block - 1) / per_block)), wblock(GACT_W8_THREADS);
+      switch (noise_mode) {
+        case GACT_NOISE_CONST:
+          hipLaunchKernelGGL((quantize_wave8_kernel<T, GACT_NOISE_CONST>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
+          break;
+        case GACT_NOISE_INJECT:
+          hipLaunchKernelGGL((quantize_wave8_kernel<T, GACT_NOISE_INJECT>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
+          break;
+        case GACT_NOISE_FAST:
+          hipLaunchKernelGGL((quantize_wave8_kernel<T, GACT_NOISE_FAST>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
+          break;
+        default:
+          return GACT_EINVAL;
+      }
+      return launch_status();
+    }
+  }
   const int sgr = noise_mode == GACT_NOISE_REF ? 1 : G.sgr;
   row_grid((supergroups(N, BITS) + sgr - 1) / sgr, &grid, &block, G.threads);
   // the reference stream's one Philox block per byte makes the kernel instruction-bound: it wants every wave
