@@ -2363,113 +2363,109 @@ inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
 #define GACT_W8_THREADS 256
 #endif
 
-// the kernel of a noise mode; its small-tensor form where the geometry has one (staging is for fused min/max and
-// not for the reference stream)
+// What a single-tensor launch is made of: the kernel, its grid, and the dynamic LDS it asks for.  Planning and
+// launching are separate so that gact_launch_geometry reports exactly what a launch would use.
+struct LaunchPlan {
+  const void* kernel = nullptr;   // null: the arguments name no kernel (an unknown noise mode or width)
+  dim3 grid, block;
+  unsigned lds = 0;
+};
+
+// the quantize kernel of a noise mode: its small-tensor form where the geometry has one (staging is for fused
+// min/max and not for the reference stream)
 template <typename T, int BITS, int NOISE, bool GIVEN>
-void launch_quantize_kernel(bool small, dim3 grid, dim3 block, unsigned lds, hipStream_t stream, const T* x, int64_t numel,
-                            int64_t N, uint8_t* packed, typename Elem<T>::Stat* scale, T* mn, T* mx, SeedArg seed,
-                            const float* noise) {
+const void* quantize_kernel_of(bool small) {
   constexpr QGeom G = q_geom<T>(BITS);
   if constexpr (!GIVEN && NOISE != GACT_NOISE_REF && (G.stage_small != G.stage || G.lazy_small != G.lazy)) {
-    if (small) {
-      hipLaunchKernelGGL((quantize_kernel<T, BITS, NOISE, GIVEN, true>), grid, block, lds, stream, x, numel, N, packed,
-                         scale, mn, mx, seed, noise);
-      return;
-    }
+    if (small) return (const void*)quantize_kernel<T, BITS, NOISE, GIVEN, true>;
   }
-  hipLaunchKernelGGL((quantize_kernel<T, BITS, NOISE, GIVEN, false>), grid, block, lds, stream, x, numel, N, packed, scale,
-                     mn, mx, seed, noise);
+  return (const void*)quantize_kernel<T, BITS, NOISE, GIVEN, false>;
 }
 
 template <typename T, int BITS, bool GIVEN>
-int launch_quantize(const T* x, int64_t numel, int64_t N, uint8_t* packed, typename Elem<T>::Stat* scale, T* mn, T* mx,
-                    int noise_mode,
-                    SeedArg seed, const float* noise, hipStream_t stream) {
-  dim3 grid, block;
+LaunchPlan plan_quantize(int64_t N, int noise_mode) {
+  LaunchPlan p;
   constexpr QGeom G = q_geom<T>(BITS);
   if constexpr (!GIVEN && BITS == 1) {
     if (noise_mode != GACT_NOISE_REF && N < (sizeof(T) == 4 ? GACT_W8_BELOW_F32 : GACT_W8_BELOW_F16)) {
       const unsigned per_block = GACT_W8_THREADS / 64;
-      const dim3 wgrid((unsigned)(((N + 7) / 8 + per_block - 1) / per_block)), wblock(GACT_W8_THREADS);
+      p.grid = dim3((unsigned)(((N + 7) / 8 + per_block - 1) / per_block));
+      p.block = dim3(GACT_W8_THREADS);
       switch (noise_mode) {
-        case GACT_NOISE_CONST:
-          hipLaunchKernelGGL((quantize_wave8_kernel<T, GACT_NOISE_CONST>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
-          break;
-        case GACT_NOISE_INJECT:
-          hipLaunchKernelGGL((quantize_wave8_kernel<T, GACT_NOISE_INJECT>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
-          break;
-        case GACT_NOISE_FAST:
-          hipLaunchKernelGGL((quantize_wave8_kernel<T, GACT_NOISE_FAST>), wgrid, wblock, 0, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
-          break;
-        default:
-          return GACT_EINVAL;
+        case GACT_NOISE_CONST: p.kernel = (const void*)quantize_wave8_kernel<T, GACT_NOISE_CONST>; break;
+        case GACT_NOISE_INJECT: p.kernel = (const void*)quantize_wave8_kernel<T, GACT_NOISE_INJECT>; break;
+        case GACT_NOISE_FAST: p.kernel = (const void*)quantize_wave8_kernel<T, GACT_NOISE_FAST>; break;
       }
-      return launch_status();
+      return p;
     }
   }
   const int sgr = noise_mode == GACT_NOISE_REF ? 1 : G.sgr;
-  row_grid((supergroups(N, BITS) + sgr - 1) / sgr, &grid, &block, G.threads);
+  row_grid((supergroups(N, BITS) + sgr - 1) / sgr, &p.grid, &p.block, G.threads);
   // the reference stream's one Philox block per byte makes the kernel instruction-bound: it wants every wave
-  const unsigned lds = noise_mode == GACT_NOISE_REF ? 0u : quantize_lds_cap(sizeof(T), BITS, N);
+  p.lds = noise_mode == GACT_NOISE_REF ? 0u : quantize_lds_cap(sizeof(T), BITS, N);
   const bool small = N < G.small_below;
   switch (noise_mode) {
-    case GACT_NOISE_CONST:
-      launch_quantize_kernel<T, BITS, GACT_NOISE_CONST, GIVEN>(small, grid, block, lds, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
-      break;
-    case GACT_NOISE_INJECT:
-      launch_quantize_kernel<T, BITS, GACT_NOISE_INJECT, GIVEN>(small, grid, block, lds, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
-      break;
-    case GACT_NOISE_REF:
-      launch_quantize_kernel<T, BITS, GACT_NOISE_REF, GIVEN>(small, grid, block, lds, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
-      break;
-    case GACT_NOISE_FAST:
-      launch_quantize_kernel<T, BITS, GACT_NOISE_FAST, GIVEN>(small, grid, block, lds, stream, x, numel, N, packed, scale, mn, mx, seed, noise);
-      break;
-    default:
-      return GACT_EINVAL;
+    case GACT_NOISE_CONST: p.kernel = quantize_kernel_of<T, BITS, GACT_NOISE_CONST, GIVEN>(small); break;
+    case GACT_NOISE_INJECT: p.kernel = quantize_kernel_of<T, BITS, GACT_NOISE_INJECT, GIVEN>(small); break;
+    case GACT_NOISE_REF: p.kernel = quantize_kernel_of<T, BITS, GACT_NOISE_REF, GIVEN>(small); break;
+    case GACT_NOISE_FAST: p.kernel = quantize_kernel_of<T, BITS, GACT_NOISE_FAST, GIVEN>(small); break;
   }
-  return launch_status();
+  return p;
 }
 
+template <typename T, bool GIVEN>
+LaunchPlan plan_quantize_bits(int bits, int64_t N, int noise_mode) {
+  switch (bits) {
+    case 1: return plan_quantize<T, 1, GIVEN>(N, noise_mode);
+    case 2: return plan_quantize<T, 2, GIVEN>(N, noise_mode);
+    case 4: return plan_quantize<T, 4, GIVEN>(N, noise_mode);
+    case 8: return plan_quantize<T, 8, GIVEN>(N, noise_mode);
+  }
+  return LaunchPlan();
+}
+
+// every quantize kernel takes the same arguments
 template <typename T, bool GIVEN>
 int dispatch_quantize(int bits, const T* x, int64_t numel, int64_t N, uint8_t* packed, typename Elem<T>::Stat* scale,
                       T* mn, T* mx,
                       int noise_mode, SeedArg seed, const float* noise, hipStream_t stream) {
-  switch (bits) {
-    case 1: return launch_quantize<T, 1, GIVEN>(x, numel, N, packed, scale, mn, mx, noise_mode, seed, noise, stream);
-    case 2: return launch_quantize<T, 2, GIVEN>(x, numel, N, packed, scale, mn, mx, noise_mode, seed, noise, stream);
-    case 4: return launch_quantize<T, 4, GIVEN>(x, numel, N, packed, scale, mn, mx, noise_mode, seed, noise, stream);
-    case 8: return launch_quantize<T, 8, GIVEN>(x, numel, N, packed, scale, mn, mx, noise_mode, seed, noise, stream);
-  }
-  return GACT_EINVAL;
+  const LaunchPlan p = plan_quantize_bits<T, GIVEN>(bits, N, noise_mode);
+  if (!p.kernel) return GACT_EINVAL;
+  void* args[] = {(void*)&x, (void*)&numel, (void*)&N, (void*)&packed, (void*)&scale, (void*)&mn, (void*)&mx, (void*)&seed, (void*)&noise};
+  return hipLaunchKernel(p.kernel, p.grid, p.block, args, p.lds, stream) == hipSuccess ? GACT_OK : GACT_ELAUNCH;
 }
 
 template <typename T>
-int dispatch_dequantize(int bits, const uint8_t* packed, const typename Elem<T>::Stat* scale, const T* mn,
-                        int64_t numel, int64_t N, T* out,
-                        hipStream_t stream) {
+LaunchPlan plan_dequantize(int bits, int64_t N) {
+  LaunchPlan p;
   // a unit takes 256 / (16 / sizeof(T)) lanes
   const DqGeom d = dq_geom<T>(bits);
   const bool large = N >= d.large_from;
   const int64_t units_per_block = d.threads / (GROUP / (16 / (int64_t)sizeof(T)));
   const int64_t unit_groups = dq_unit_groups(d, bits, large);
   // the caps are stated for workgroups of 256 threads
-  const unsigned lds = large ? d.lds_large * (unsigned)d.threads / 256u : 0u;
-  const dim3 grid((unsigned)(((N + unit_groups - 1) / unit_groups + units_per_block - 1) / units_per_block)), block((unsigned)d.threads);
-#define GACT_LAUNCH_DQ(B)                                                                                              \
-  if (large)                                                                                                           \
-    hipLaunchKernelGGL((dequantize_kernel<T, B, true>), grid, block, lds, stream, packed, scale, mn, numel, N, out);  \
-  else                                                                                                                 \
-    hipLaunchKernelGGL((dequantize_kernel<T, B, false>), grid, block, lds, stream, packed, scale, mn, numel, N, out)
+  p.lds = large ? d.lds_large * (unsigned)d.threads / 256u : 0u;
+  p.grid = dim3((unsigned)(((N + unit_groups - 1) / unit_groups + units_per_block - 1) / units_per_block));
+  p.block = dim3((unsigned)d.threads);
+#define GACT_DQ_KERNEL(B) (large ? (const void*)dequantize_kernel<T, B, true> : (const void*)dequantize_kernel<T, B, false>)
   switch (bits) {
-    case 1: GACT_LAUNCH_DQ(1); break;
-    case 2: GACT_LAUNCH_DQ(2); break;
-    case 4: GACT_LAUNCH_DQ(4); break;
-    case 8: GACT_LAUNCH_DQ(8); break;
-    default: return GACT_EINVAL;
+    case 1: p.kernel = GACT_DQ_KERNEL(1); break;
+    case 2: p.kernel = GACT_DQ_KERNEL(2); break;
+    case 4: p.kernel = GACT_DQ_KERNEL(4); break;
+    case 8: p.kernel = GACT_DQ_KERNEL(8); break;
   }
-#undef GACT_LAUNCH_DQ
-  return launch_status();
+#undef GACT_DQ_KERNEL
+  return p;
+}
+
+template <typename T>
+int dispatch_dequantize(int bits, const uint8_t* packed, const typename Elem<T>::Stat* scale, const T* mn,
+                        int64_t numel, int64_t N, T* out,
+                        hipStream_t stream) {
+  const LaunchPlan p = plan_dequantize<T>(bits, N);
+  if (!p.kernel) return GACT_EINVAL;
+  void* args[] = {(void*)&packed, (void*)&scale, (void*)&mn, (void*)&numel, (void*)&N, (void*)&out};
+  return hipLaunchKernel(p.kernel, p.grid, p.block, args, p.lds, stream) == hipSuccess ? GACT_OK : GACT_ELAUNCH;
 }
 
 template <typename T>
@@ -2684,6 +2680,29 @@ int gact_dequantize(const void* packed, int bits, const void* scale, const void*
   if (dtype == GACT_BF16)
     return dispatch_dequantize<bf16>(bits, (const uint8_t*)packed, (const float*)scale, (const bf16*)mn, numel, N, (bf16*)out, s);
   return dispatch_dequantize<f16>(bits, (const uint8_t*)packed, (const f16*)scale, (const f16*)mn, numel, N, (f16*)out, s);
+}
+
+int gact_launch_geometry(int kind, int dtype, int bits, int64_t N, int* threads, int* lds_bytes, int* workgroups_per_cu) {
+  if (dtype != GACT_F32 && dtype != GACT_F16 && dtype != GACT_BF16) return GACT_EINVAL;
+  if (!valid_bits(bits) || N <= 0 || (kind != 0 && kind != 1)) return GACT_EINVAL;
+  LaunchPlan p;
+  if (kind == 0)
+    p = dtype == GACT_F32 ? plan_quantize_bits<float, false>(bits, N, GACT_NOISE_FAST)
+        : dtype == GACT_F16 ? plan_quantize_bits<f16, false>(bits, N, GACT_NOISE_FAST)
+                            : plan_quantize_bits<bf16, false>(bits, N, GACT_NOISE_FAST);
+  else
+    p = dtype == GACT_F32 ? plan_dequantize<float>(bits, N)
+        : dtype == GACT_F16 ? plan_dequantize<f16>(bits, N) : plan_dequantize<bf16>(bits, N);
+  if (!p.kernel) return GACT_EINVAL;
+  int per_cu = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, p.kernel, (int)p.block.x, (size_t)p.lds) != hipSuccess) {
+    (void)hipGetLastError();
+    return GACT_ELAUNCH;
+  }
+  if (threads) *threads = (int)p.block.x;
+  if (lds_bytes) *lds_bytes = (int)p.lds;
+  if (workgroups_per_cu) *workgroups_per_cu = per_cu;
+  return GACT_OK;
 }
 
 int gact_mask_pack(const uint8_t* data, int64_t n, int32_t* mask, void* stream) {

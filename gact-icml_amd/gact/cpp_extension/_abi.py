@@ -15,7 +15,7 @@ F32, F16, BF16 = 0, 1, 2
 NOISE_CONST, NOISE_INJECT, NOISE_REF, NOISE_FAST = 0, 1, 2, 3
 NOISE_MODES = {"deterministic": NOISE_CONST, "inject": NOISE_INJECT, "reference": NOISE_REF, "fast": NOISE_FAST}
 GROUP = 256
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 
 class BatchEntry(ctypes.Structure):
@@ -46,6 +46,7 @@ SIGNATURES = {
     "gact_quantize": (_i32, [_vp, _i32, _i64, _i32, _i32, _u64, _vp, _vp, _vp, _vp, _vp, _vp]),
     "gact_quantize_seeded": (_i32, [_vp, _i32, _i64, _i32, _i32, _u64, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "gact_dequantize": (_i32, [_vp, _i32, _vp, _vp, _i32, _i64, _vp, _vp]),
+    "gact_launch_geometry": (_i32, [_i32, _i32, _i32, _i64, _vp, _vp, _vp]),
     "gact_mask_pack": (_i32, [_vp, _i64, _vp, _vp]),
     "gact_mask_unpack": (_i32, [_vp, _i64, _vp, _vp]),
     "gact_calc_precision": (_i32, [_vp, _vp, _vp, _i64, _f64]),

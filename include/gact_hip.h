@@ -17,7 +17,7 @@
 extern "C" {
 #endif
 
-#define GACT_ABI_VERSION 6
+#define GACT_ABI_VERSION 7
 
 /* element types of activations, min, max and scale */
 #define GACT_F32 0
@@ -89,6 +89,14 @@ int gact_quantize_seeded(const void* x, int dtype, int64_t numel, int bits, int 
  * group size 256: writes exactly `numel` elements. */
 int gact_dequantize(const void* packed, int bits, const void* scale, const void* mn, int dtype,
                     int64_t numel, void* out, void* stream);
+
+/* What a gact_quantize (kind 0; fast, deterministic or injected noise) or gact_dequantize (kind 1) launch of a tensor of
+ * N groups is made of, without launching anything: the threads of a workgroup, the dynamic LDS the launch asks for -
+ * on large tensors some kernels ask for LDS they never touch, which is how the library caps their occupancy - and
+ * the workgroups of that kernel a compute unit holds under both (hipOccupancyMaxActiveBlocksPerMultiprocessor).
+ * Any of the three pointers may be null.  No counterpart in the reference; for tests and tuning. */
+int gact_launch_geometry(int kind, int dtype, int bits, int64_t N, int* threads, int* lds_bytes,
+                         int* workgroups_per_cu);
 
 /* Dropout-mask bit packing: n bytes (nonzero = 1) <-> ceil(n/32) int32 words.
  * Replace act_quantize_dropout_mask_cuda / act_dequantize_dropout_mask_cuda

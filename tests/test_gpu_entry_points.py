@@ -359,3 +359,50 @@ def test_random_cases_on_general_shapes_masks_and_minimax():
             x = buf[off:].view(N, D)
             mn, mx = ext_minimax.minimax(x)
             assert torch.equal(mn, x.min(1).values) and torch.equal(mx, x.max(1).values), (N, D, off, dtype)
+
+
+def test_occupancy_caps_are_what_the_launches_get():
+    """On large tensors some kernels cap their occupancy by asking for dynamic LDS they never touch.  What the
+    runtime grants for exactly the kernel, workgroup size and LDS request of a launch (gact_launch_geometry:
+    hipOccupancyMaxActiveBlocksPerMultiprocessor) must be the cap the geometry tables mean - and no cap where
+    none is meant."""
+    import ctypes
+
+    lib = _abi.lib()
+
+    def geometry(kind, dtype, bits, N):
+        t, l, w = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+        _abi.check(lib.gact_launch_geometry(kind, dtype, bits, N, ctypes.addressof(t), ctypes.addressof(l), ctypes.addressof(w)))
+        return t.value, l.value, w.value
+
+    Q, DQ = 0, 1
+    big, small = 1 << 19, 1 << 14
+    # dequantize, float, every width: 3 workgroups of 256 threads per compute unit from 2^17 groups on
+    for bits in (1, 2, 4, 8):
+        threads, lds, per_cu = geometry(DQ, _abi.F32, bits, big)
+        assert (threads, per_cu) == (256, 3) and lds > 0, (bits, threads, lds, per_cu)
+        threads, lds, per_cu = geometry(DQ, _abi.F32, bits, small)
+        assert threads == 256 and lds == 0 and per_cu >= 6, (bits, per_cu)
+    # dequantize, half: capped at 8 bit only (4 workgroups)
+    assert geometry(DQ, _abi.F16, 8, big)[1:] == (40000, 4)
+    for bits in (1, 2, 4):
+        assert geometry(DQ, _abi.F16, bits, big)[1] == 0 and geometry(DQ, _abi.F16, bits, big)[2] >= 6
+    # quantize, float: 16 one-wave workgroups per compute unit at 4 bit, 8 at 2 bit, on large tensors only
+    assert geometry(Q, _abi.F32, 4, big) == (64, 10000, 16)
+    assert geometry(Q, _abi.F32, 2, big) == (64, 20000, 8)
+    assert geometry(Q, _abi.F32, 4, small)[1] == 0 and geometry(Q, _abi.F32, 2, small)[1] == 0
+    for bits in (1, 8):
+        assert geometry(Q, _abi.F32, bits, big)[1] == 0
+    for dtype in (_abi.F16, _abi.BF16):
+        for bits in (1, 2, 4, 8):
+            assert geometry(Q, dtype, bits, big)[1] == 0
+    # uncapped one-wave workgroups: the registers decide (float 1 bit holds 8 groups per lane: two waves per SIMD)
+    assert geometry(Q, _abi.F32, 1, big)[0] == 64 and geometry(Q, _abi.F32, 1, big)[2] >= 8
+    # small 1-bit tensors take the wave-per-super-group kernel, four waves to a workgroup
+    assert geometry(Q, _abi.F32, 1, small)[0] == 256 and geometry(Q, _abi.F16, 1, small)[0] == 256
+    # arguments
+    assert lib.gact_launch_geometry(2, _abi.F32, 4, 100, None, None, None) == -1
+    assert lib.gact_launch_geometry(0, _abi.F32, 3, 100, None, None, None) == -1
+    assert lib.gact_launch_geometry(0, 7, 4, 100, None, None, None) == -1
+    assert lib.gact_launch_geometry(1, _abi.F16, 4, 0, None, None, None) == -1
+    assert lib.gact_launch_geometry(1, _abi.F16, 4, 100, None, None, None) == 0

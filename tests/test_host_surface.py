@@ -42,7 +42,7 @@ def test_struct_layout_matches_the_header():
 
 def test_status_codes_and_sizes():
     L = _abi.lib()
-    assert L.gact_abi_version() == 6
+    assert L.gact_abi_version() == 7
     assert L.gact_strerror(0) == b"ok"
     for code in (-1, -2, -3, -4, -5):
         assert L.gact_strerror(code) not in (b"ok", b"unknown error")
