@@ -17,6 +17,10 @@ each kernel comes from the same construction with K launches of that kernel alon
 slower of the two kernels of the headline workload.  `cpu_baseline` is the C restatement of the reference
 arithmetic (oracle/) with OpenMP on the host cores.
 
+Every workload also carries `probe`: compute-free kernels (gact-icml_amd/csrc/stream_probe.hip) that move the bytes of
+its quantize and of its dequantize kernel - the same bytes per wave in, the same out, nothing computed - timed the same
+way in the same run, and the kernel's duration as a multiple of the probe's.
+
 Beside the workloads the line carries what plain streams reach in the same run: `ceilings` (device copy, fill,
 pure read, torch's element-wise kernel at the 8:1 and 1:8 read:write mixes, and the duration of a one-group
 launch, on config2's tensor), `ceilings_headline` (the same on config1's tensor) and `ceilings_by_size` (fill and
@@ -68,6 +72,8 @@ WORKLOADS = {
     "config3-hidden": ((16384, 1024), "float16", 8, "fast", "randn", "BERT-large hidden states fp16, 8 bit"),
     "config3-gelu": ((16384, 4096), "float16", 4, "fast", "randn", "BERT-large GELU inputs fp16, 4 bit"),
     "config3-probs": ((32, 16, 512, 512), "float16", 2, "fast", "softmax", "BERT-large attention probs fp16, 2 bit"),
+    "config3-probs-refstream": ((32, 16, 512, 512), "float16", 2, "reference", "softmax",
+                                "config3's attention probs with the reference's one-Philox-state-per-byte noise stream"),
     "config4": ((169343, 256), "float32", 1, "fast", "relu60", "GCN node features fp32 [169343,256], ~60% zeros, 1 bit"),
     # the reference's own micro-benchmark (tests/test_speed.py:6-15): torch.rand [256,256,14,14] at 2 bit
     "reference-test-speed": ((256, 256, 14, 14), "float32", 2, "fast", "rand",
@@ -76,8 +82,8 @@ WORKLOADS = {
     "bf16-gelu": ((16384, 4096), "bfloat16", 4, "fast", "randn", "GELU inputs in bfloat16, 4 bit (float scale, bfloat16 min)"),
 }
 # what a default run measures besides the headline workload (config5 is the batched one)
-BASELINE_SET = ["config1", "config2", "config2-2bit", "config3-hidden", "config3-gelu", "config3-probs", "config4",
-                "reference-test-speed"]
+BASELINE_SET = ["config1", "config2", "config2-refstream", "config2-2bit", "config3-hidden", "config3-gelu", "config3-probs",
+                "config3-probs-refstream", "config4", "reference-test-speed"]
 
 
 def make_input(torch, shape, dtype, kind, seed=0):
@@ -99,6 +105,25 @@ def algorithmic_bytes(numel, esize, bits, scale_esize=None):
     wpt = 8 // bits
     n_round = (N + wpt - 1) // wpt * wpt
     return numel * esize + n_round * 32 * bits + N * (esize + (scale_esize or esize))
+
+
+_PROBE = None
+
+
+def probe_lib():
+    """The compute-free traffic probes (libgact_probe.so, built next to the library)."""
+    global _PROBE
+    if _PROBE is None:
+        import ctypes
+
+        from gact.cpp_extension import _abi
+        lib = ctypes.CDLL(os.path.join(os.path.dirname(_abi.LIB_PATH), "libgact_probe.so"))
+        vp, i32, i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
+        for name in ("gact_probe_quantize_like", "gact_probe_dequantize_like"):
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = i32, [vp, vp, i64, i32, i32, vp]
+        _PROBE = lib
+    return _PROBE
 
 
 class Timer:
@@ -196,6 +221,31 @@ def run_workload(torch, name, timer, seed=42, keep_input=False, rotate=True):
     q_ms, _ = timer(quantize, sets)
     d_ms, _ = timer(dequantize, sets)
 
+    # the same traffic without the arithmetic: a wave reads 8 groups (8 KB float, 4 KB half) and writes their 256 * bits
+    # bytes of codes, or the reverse - into the very buffers the kernels use (scale and min, under 1 % of the bytes,
+    # are left out)
+    probe = probe_lib()
+    kb = 8 if esize == 4 else 4
+    whole = numel * esize // (kb * 1024)
+
+    def quantize_like(k):
+        xi, packed, _, _, _ = bufs[k % sets]
+        rc = probe.gact_probe_quantize_like(xi.data_ptr(), packed.data_ptr(), numel * esize, kb, bits,
+                                            torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+
+    def dequantize_like(k):
+        _, packed, _, _, out = bufs[k % sets]
+        rc = probe.gact_probe_dequantize_like(packed.data_ptr(), out.data_ptr(), numel * esize, bits, kb,
+                                              torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+
+    pq_ms, _ = timer(quantize_like, sets)
+    pd_ms, _ = timer(dequantize_like, sets)
+    probe_bytes = whole * (kb * 1024 + 256 * bits)
+    for k in range(sets):   # the probes overwrote codes and outputs: leave every set as the kernels left it
+        step(k)
+
     per_dir = algorithmic_bytes(numel, esize, bits, 4 if x.dtype == torch.bfloat16 else None)
     gbs = lambda ms: per_dir / (ms * 1e-3) / 1e9
     res = {
@@ -204,6 +254,12 @@ def run_workload(torch, name, timer, seed=42, keep_input=False, rotate=True):
         "gbs": 2 * per_dir / (step_ms * 1e-3) / 1e9,
         "quantize": {"ms": q_ms, "gbs": gbs(q_ms)},
         "dequantize": {"ms": d_ms, "gbs": gbs(d_ms)},
+        "probe": {"what": "compute-free kernels with the traffic of the two kernels (%d KB and %d bytes per wave)" % (kb, 256 * bits),
+                  "bytes": probe_bytes,
+                  "quantize_like": {"us": pq_ms * 1e3, "frac": probe_bytes / (pq_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                    "kernel_over_probe": q_ms / pq_ms},
+                  "dequantize_like": {"us": pd_ms * 1e3, "frac": probe_bytes / (pd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                      "kernel_over_probe": d_ms / pd_ms}},
     }
     return res, (x if keep_input else None)
 
@@ -404,13 +460,14 @@ def python_ops_us(torch, name, min_seconds):
 def compact(res):
     """The per-configuration entry of the JSON line."""
     out = {
-        "desc": res["desc"], "dtype": res["dtype"], "bits": res["bits"], "bytes_per_direction": res["bytes_per_direction"],
+        "desc": res["desc"], "dtype": res["dtype"], "bits": res["bits"], "rng_stream": res["rng_stream"],
+        "bytes_per_direction": res["bytes_per_direction"],
         "buffer_sets": res["buffer_sets"],
         "step": {"us": res["ms_per_step"] * 1e3, "gbs": res["gbs"], "frac": res["gbs"] / HBM_PEAK_GBS},
     }
     for k in ("quantize", "dequantize"):
         out[k] = {"us": res[k]["ms"] * 1e3, "gbs": res[k]["gbs"], "frac": res[k]["gbs"] / HBM_PEAK_GBS}
-    for k in ("width_histogram", "tensors", "elements"):
+    for k in ("width_histogram", "tensors", "elements", "probe"):
         if k in res:
             out[k] = res[k]
     if "calc_precision" in res:

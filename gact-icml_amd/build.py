@@ -1,4 +1,5 @@
-"""Build libgact_hip.so (the C-ABI library of HIP kernels) for gfx950 with hipcc.
+"""Build libgact_hip.so (the C-ABI library of HIP kernels) and libgact_probe.so (compute-free traffic probes that
+bench.py measures beside the kernels) for gfx950 with hipcc.
 
     python gact-icml_amd/build.py            # build if the sources are newer than the library
     python gact-icml_amd/build.py --force
@@ -14,9 +15,11 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 SRC = os.path.join(HERE, "csrc", "gact_hip.hip")
+PROBE_SRC = os.path.join(HERE, "csrc", "stream_probe.hip")   # compute-free traffic probes for bench.py
 HDR = os.path.join(ROOT, "include", "gact_hip.h")
 OUT_DIR = os.path.join(HERE, "gact", "lib")
 OUT = os.path.join(OUT_DIR, "libgact_hip.so")
+PROBE_OUT = os.path.join(OUT_DIR, "libgact_probe.so")
 
 HIPCC_FLAGS = [
     "-O3",
@@ -41,10 +44,10 @@ def hipcc():
 
 
 def up_to_date():
-    if not os.path.exists(OUT):
+    if not os.path.exists(OUT) or not os.path.exists(PROBE_OUT):
         return False
-    t = os.path.getmtime(OUT)
-    return all(os.path.getmtime(p) <= t for p in (SRC, HDR, os.path.abspath(__file__)))
+    t = min(os.path.getmtime(OUT), os.path.getmtime(PROBE_OUT))
+    return all(os.path.getmtime(p) <= t for p in (SRC, PROBE_SRC, HDR, os.path.abspath(__file__)))
 
 
 def build(force=False, extra=()):
@@ -53,6 +56,7 @@ def build(force=False, extra=()):
     os.makedirs(OUT_DIR, exist_ok=True)
     cmd = [hipcc()] + HIPCC_FLAGS + list(extra) + ["-I", os.path.join(ROOT, "include"), "-o", OUT, SRC]
     subprocess.run(cmd, check=True)
+    subprocess.run([hipcc()] + HIPCC_FLAGS + ["-o", PROBE_OUT, PROBE_SRC], check=True)
     return OUT
 
 

@@ -1420,45 +1420,46 @@ __device__ __forceinline__ uint32_t pack4(const uint32_t* b) {
   // the reference accumulates in a uint8_t: keep the low 8 bits of every byte
   return (b[0] & 0xffu) | ((b[1] & 0xffu) << 8) | ((b[2] & 0xffu) << 16) | (b[3] << 24);
 }
-template <typename T, int NOISE>
+template <typename T, int BITS, int NOISE>
 __global__ void __launch_bounds__(256)
 quantize_wave8_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __restrict__ packed,
                       typename Elem<T>::Stat* __restrict__ scale_out, T* __restrict__ mn_out, T* __restrict__ mx_out,
                       SeedArg seed_arg, const float* __restrict__ noise) {
   static_assert(NOISE != GACT_NOISE_REF, "the reference stream draws per output byte");
+  static_assert(BITS == 1 || BITS == 2, "four rows share a super-group: two groups a row at 1 bit, one at 2 bit");
   typedef typename Elem<T>::Stat Stat;
-  constexpr int BITS = 1, WPT = 8, QMAX = 1;
+  constexpr int WPT = 8 / BITS, GR = WPT / 4, QMAX = (1 << BITS) - 1;   // GR: groups of a row
   constexpr int CH = Elem<T>::kQChunks, W = Elem<T>::kQWidth;
   const uint32_t tile = gridDim.x - 1u - xcd_tile<GACT_W8_RUN>(blockIdx.x, gridDim.x);   // last tile first, see quantize_kernel
   const int64_t sg = (int64_t)tile * (blockDim.x >> 6) + (threadIdx.x >> 6);               // the wave's super-group
   const int64_t n0 = sg * WPT;
   if (n0 >= N) return;   // the whole wave
   const int lane = threadIdx.x & 63, r = lane >> 4, i = lane & 15;
-  const int64_t na = n0 + 2 * r;   // the row's groups: na, na + 1
+  const int64_t na = n0 + GR * r;   // the row's first group
   const uint64_t seed = seed_arg.value();
   const uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
 
-  typename Elem<T>::Store v[2];
+  typename Elem<T>::Store v[GR];
 #pragma unroll
-  for (int g = 0; g < 2; g++)
+  for (int g = 0; g < GR; g++)
     if (na + g < N) load_group<T>(x, numel, na + g, i, v[g]);
-  Stat lo[2], hi[2], sc[2];
+  Stat lo[GR], hi[GR], sc[GR];
 #pragma unroll
-  for (int g = 0; g < 2; g++) {
+  for (int g = 0; g < GR; g++) {
     lo[g] = hi[g] = (Stat)0.0f;
     if (na + g < N) Elem<T>::group_minmax(v[g], lo[g], hi[g]);
   }
   {
-    const bool second = i & 1;   // odd lanes divide for the row's second group
-    const Stat lo_m = second ? lo[1] : lo[0], hi_m = second ? hi[1] : hi[0];
+    const int mine = i & (GR - 1);   // with two groups a row, odd lanes divide for the second
+    const Stat lo_m = mine ? lo[GR - 1] : lo[0], hi_m = mine ? hi[GR - 1] : hi[0];
     const Stat s_m = Elem<T>::make_scale(lo_m, hi_m, QMAX);
-    if (i < 2 && na + i < N) {
+    if (i < GR && na + i < N) {
       scale_out[na + i] = s_m;
       mn_out[na + i] = Elem<T>::elem_of(lo_m);
       if (mx_out) mx_out[na + i] = Elem<T>::elem_of(hi_m);
     }
-    sc[0] = row_bcast<0>(s_m);
-    sc[1] = row_bcast<1>(s_m);
+    sc[0] = GR == 1 ? s_m : row_bcast<0>(s_m);
+    if (GR > 1) sc[GR - 1] = row_bcast<1>(s_m);
   }
 
   uint32_t bytes[CH][W];
@@ -1466,11 +1467,11 @@ quantize_wave8_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t
   for (int k = 0; k < CH; k++)
 #pragma unroll
     for (int e = 0; e < W; e++) bytes[k][e] = 0;
-  FastRow<T, 2> fast;
+  FastRow<T, GR> fast;
 #pragma unroll
-  for (int g = 0; g < 2; g++) {
+  for (int g = 0; g < GR; g++) {
     const int64_t n = na + g;
-    const uint32_t shift = (uint32_t)((2 * r + g) * BITS);   // the group's field within its bytes
+    const uint32_t shift = (uint32_t)((GR * r + g) * BITS);   // the group's field within its bytes
     if (n < N) {
       if (NOISE == GACT_NOISE_FAST) {
         float cd[CH / 2][W];
@@ -2352,7 +2353,10 @@ inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
   return 0u;
 }
 
-// Below how many groups a 1-bit quantize takes the wave-per-super-group kernel (0: never), by element size.
+// Below how many groups a 1-bit quantize takes the wave-per-super-group kernel (0: never), by element size.  (The kernel
+// also exists at 2 bit - four rows of one group each, 4 KB per float wave - and is not launched there: float [4096,1024]
+// at 2 bit, deterministic, 5.22 us with a row per super-group against 5.37-5.52 us that way, in workgroups of one or
+// four waves, with or without the XCD-aware tile order; 13 M elements 11.3 against 11.4-11.8 us; 103 M 68.1 / 67.6-68.8.)
 #ifndef GACT_W8_BELOW_F32
 #define GACT_W8_BELOW_F32 57344
 #endif
@@ -2389,12 +2393,12 @@ LaunchPlan plan_quantize(int64_t N, int noise_mode) {
   if constexpr (!GIVEN && BITS == 1) {
     if (noise_mode != GACT_NOISE_REF && N < (sizeof(T) == 4 ? GACT_W8_BELOW_F32 : GACT_W8_BELOW_F16)) {
       const unsigned per_block = GACT_W8_THREADS / 64;
-      p.grid = dim3((unsigned)(((N + 7) / 8 + per_block - 1) / per_block));
+      p.grid = dim3((unsigned)((supergroups(N, BITS) + per_block - 1) / per_block));
       p.block = dim3(GACT_W8_THREADS);
       switch (noise_mode) {
-        case GACT_NOISE_CONST: p.kernel = (const void*)quantize_wave8_kernel<T, GACT_NOISE_CONST>; break;
-        case GACT_NOISE_INJECT: p.kernel = (const void*)quantize_wave8_kernel<T, GACT_NOISE_INJECT>; break;
-        case GACT_NOISE_FAST: p.kernel = (const void*)quantize_wave8_kernel<T, GACT_NOISE_FAST>; break;
+        case GACT_NOISE_CONST: p.kernel = (const void*)quantize_wave8_kernel<T, BITS, GACT_NOISE_CONST>; break;
+        case GACT_NOISE_INJECT: p.kernel = (const void*)quantize_wave8_kernel<T, BITS, GACT_NOISE_INJECT>; break;
+        case GACT_NOISE_FAST: p.kernel = (const void*)quantize_wave8_kernel<T, BITS, GACT_NOISE_FAST>; break;
       }
       return p;
     }
