@@ -46,10 +46,20 @@ MIN_SECONDS = 1.0      # every timed loop runs at least this long
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size
 # in the same runs (profiles/<workload>_*.txt name the runs and the factors); absent = no counter run
 TRAFFIC_BYTES = {
-    ("config1", "quantize"): 18.05e6,    # 16.85 MB read + 1.20 MB written; algorithmic 17.96 MB
-    ("config1", "dequantize"): 18.02e6,  # 1.25 MB read + 16.78 MB written
-    ("config2", "quantize"): 468.90e6,   # 411.1 MB read + 57.8 MB written; algorithmic 465.6 MB
-    ("config2", "dequantize"): 465.70e6, # 54.7 MB read + 411.0 MB written
+    ("config1", "quantize"): 18.07e6,    # 16.85 MB read + 1.22 MB written; algorithmic 17.96 MB
+    ("config1", "dequantize"): 18.02e6,  # 1.25 MB read + 16.78 MB written; algorithmic 17.96 MB
+    ("config2", "quantize"): 468.31e6,    # 411.06 MB read + 57.24 MB written; algorithmic 465.63 MB
+    ("config2", "dequantize"): 465.69e6,  # 54.65 MB read + 411.04 MB written; algorithmic 465.63 MB
+    ("config3-hidden", "quantize"): 50.63e6,    # 33.59 MB read + 17.04 MB written; algorithmic 50.59 MB
+    ("config3-hidden", "dequantize"): 50.69e6,  # 17.14 MB read + 33.55 MB written; algorithmic 50.59 MB
+    ("config3-gelu", "quantize"): 168.88e6,    # 134.27 MB read + 34.60 MB written; algorithmic 168.82 MB
+    ("config3-gelu", "dequantize"): 168.88e6,  # 34.66 MB read + 134.22 MB written; algorithmic 168.82 MB
+    ("config3-probs", "quantize"): 304.20e6,    # 268.55 MB read + 35.65 MB written; algorithmic 304.09 MB
+    ("config3-probs", "dequantize"): 304.15e6,  # 35.71 MB read + 268.44 MB written; algorithmic 304.09 MB
+    ("config4", "quantize"): 180.96e6,    # 173.58 MB read + 7.38 MB written; algorithmic 180.18 MB
+    ("config4", "dequantize"): 180.34e6,  # 6.84 MB read + 173.50 MB written; algorithmic 180.18 MB
+    ("config5", "quantize"): 4143.22e6,    # 3661.83 MB read + 481.39 MB written; algorithmic 4142.23 MB
+    ("config5", "dequantize"): 4143.55e6,  # 482.71 MB read + 3660.84 MB written; algorithmic 4142.23 MB
 }
 
 BASELINE_METRIC = "quantize+dequantize GB/s and % of HBM peak, 1×MI355X, 2-bit group=256"
@@ -466,7 +476,8 @@ def compact(res):
         "step": {"us": res["ms_per_step"] * 1e3, "gbs": res["gbs"], "frac": res["gbs"] / HBM_PEAK_GBS},
     }
     for k in ("quantize", "dequantize"):
-        out[k] = {"us": res[k]["ms"] * 1e3, "gbs": res[k]["gbs"], "frac": res[k]["gbs"] / HBM_PEAK_GBS}
+        out[k] = {"us": res[k]["ms"] * 1e3, "gbs": res[k]["gbs"], "frac": res[k]["gbs"] / HBM_PEAK_GBS,
+                  "traffic": TRAFFIC_BYTES.get((res["workload"], k))}    # HBM bytes per launch by the counters, or null
     for k in ("width_histogram", "tensors", "elements", "probe"):
         if k in res:
             out[k] = res[k]
@@ -531,15 +542,18 @@ def main():
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get((args.workload, dom))},
     }
-    if args.copy_calibration and x is not None:
-        y = torch.empty_like(x)
+    if args.copy_calibration:
+        # a copy kernel of known size for a counter run to scale by: the workload's tensor, or 256 MiB where the
+        # workload has no single tensor (config5)
+        src = x if x is not None else torch.zeros((1 << 28,), dtype=torch.uint8, device="cuda")
+        y = torch.empty_like(src)
         for _ in range(20):
-            y.copy_(x)
+            y.copy_(src)
         torch.cuda.synchronize()
-        line["copy_calibration"] = {"kernel": "torch elementwise copy", "launches": 20,
-                                    "bytes_read": x.numel() * x.element_size(),
-                                    "bytes_written": x.numel() * x.element_size()}
-        del y
+        line["copy_calibration"] = {"kernel": "device-to-device copy", "launches": 20,
+                                    "bytes_read": src.numel() * src.element_size(),
+                                    "bytes_written": src.numel() * src.element_size()}
+        del y, src
     if not args.only:
         configs = {args.workload: compact(res)}
         for name in BASELINE_SET + ["config5"]:
