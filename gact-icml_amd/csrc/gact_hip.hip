@@ -1063,8 +1063,8 @@ __device__ __forceinline__ void dequantize_unit(const uint8_t* __restrict__ pack
     // instruction each, a handful of lanes active - and the table entries fetch theirs across the unit.  Letting every
     // entry load its own (2 * PASSES instructions, all lanes active, for a fraction of a percent of the bytes) cost the
     // single-tensor kernel 7 % at half 4 bit (67 M elements 30.3 -> 28.2 us) and 4 % at half 2 bit (134 M: 50.5 -> 48.5);
-    // the batched launch, whose half units are 8 groups, is within 2 % either way at 1 bit and loses 3 % at 2 bit and 7 % at
-    // 4 bit by sharing (120 tensors, 1.83 G elements: 648 -> 633, 683 -> 705, 757 -> 812 us), so its entries load their own.
+    // with half units of 8 groups sharing loses instead (the batched launch when it had such units: 2 bit 683 -> 705 us,
+    // 4 bit 757 -> 812 for 1.83 G elements), and float units, a whole wave each, are within 1 % either way.
     const uint32_t unitbase = (threadIdx.x & 63u) & ~(uint32_t)(LPU - 1);  // first lane of the unit within its wave
     uint32_t tab[PASSES];
     if constexpr (SHARE_STATS) {
@@ -1226,21 +1226,27 @@ __device__ __forceinline__ void quantize_block128(const T* __restrict__ x, int64
                                                                     (uint32_t)seed, (uint32_t)(seed >> 32), nullptr);
   }
 }
-// Dequantize: two workgroups share a block of 128 groups, 8 units of 8 groups each, so that a unit slot
-// (a wave for float, half a wave for half) gets one unit for half and two for float - several units in a
-// row per wave cost 10-20 %.
+// Dequantize: four workgroups share a block of 128 groups, 32 groups each - 4 units of 8 groups for float (a wave
+// each), 8 units of 4 groups for half and bfloat16 (half a wave each; at 1 bit a unit is half a super-group and two
+// units load the same code words): one unit per slot, several in a row per wave cost 10-20 %.  Half units of 4 groups
+// with their scale and min shared across the unit are what the single-tensor kernel prefers on tensors of this size;
+// against two workgroups per block and half units of 8 groups (120 half tensors, 1.83 G elements, all at one width):
+// 2 bit 696 -> 677 us, 4 bit 758 -> 732, 8 bit 937 -> 929, 1 bit 651 -> 683; a mix of widths 719 -> 687.
 template <typename T, int BITS>
 __device__ __forceinline__ void dequantize_block128(const uint8_t* __restrict__ packed,
                                                     const typename Elem<T>::Stat* __restrict__ scale,
                                                     const T* __restrict__ mn, int64_t numel, int64_t N, int64_t lb,
-                                                    int half, T* __restrict__ out) {
+                                                    int quarter, T* __restrict__ out) {
   constexpr int LPU = GROUP / Elem<T>::kDqWidth;  // lanes per unit
-  constexpr int SLOTS = 256 / LPU;
+  constexpr int SLOTS = 256 / LPU;                // units of the workgroup
   const int slot = threadIdx.x / LPU, l = threadIdx.x % LPU;
-#pragma unroll 1
-  for (int it = 0; it < 8 / SLOTS; it++) {
-    const int64_t unit = lb * 16 + half * 8 + it * SLOTS + slot;
-    if (unit * ROW_GROUPS < N) dequantize_unit<T, BITS, BITS, 1, true, false>(packed, scale, mn, numel, N, unit, l, out);
+  if constexpr (LPU == 64) {
+    const int64_t unit = lb * 16 + quarter * SLOTS + slot;   // units of 8 groups
+    if (unit * 8 < N) dequantize_unit<T, BITS, BITS, 1, true, false>(packed, scale, mn, numel, N, unit, l, out);
+  } else {
+    const int64_t unit = lb * 32 + quarter * SLOTS + slot;   // units of 4 groups
+    constexpr int SGS = BITS == 1 ? 1 : BITS / 2, PARTS = BITS == 1 ? 2 : 1;
+    if (unit * 4 < N) dequantize_unit<T, BITS, SGS, PARTS, true, true>(packed, scale, mn, numel, N, unit, l, out);
   }
 }
 
@@ -2275,16 +2281,16 @@ __device__ __forceinline__ void dequantize_batched_block(const gact_batch_entry&
   else
     dequantize_block128<bf16, BITS>(packed, (const float*)sc, (const bf16*)mn, ent.numel, N, lb, half, (bf16*)ent.x);
 }
-// grid: two workgroups per block of 128 groups
+// grid: four workgroups per block of 128 groups
 __global__ void __launch_bounds__(256)
 dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_t* __restrict__ bits,
                           BatchWorkspace ws, const uint8_t* __restrict__ packed_arena,
                           const uint8_t* __restrict__ scale_arena, const uint8_t* __restrict__ min_arena) {
   if (ws.hdr->ok == 0) return;
-  // half a block is the single-tensor kernel's tile; same XCD-aware order (715 -> 709 us on 120 half tensors)
+  // the XCD-aware order of the single-tensor kernel (715 -> 709 us on 120 half tensors)
   const uint32_t tile = xcd_tile<GACT_XCD_RUN_DQB>(blockIdx.x, gridDim.x);
-  const int64_t block = tile >> 1;
-  const int half = tile & 1;
+  const int64_t block = tile >> 2;
+  const int half = tile & 3;   // which quarter of the block
   const int t = ws.block_tensor[block];
   const gact_batch_entry ent = table[t];
   const int64_t lb = block - ent.first_block;
@@ -2856,8 +2862,9 @@ int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, 
   if (L == 0 || total_blocks == 0) return GACT_OK;
   if (!table || !bits || !workspace || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena) || !aligned16(workspace)) return GACT_EALIGN;
+  if (total_blocks > 0x1fffffffLL) return GACT_EINVAL;   // four workgroups per block must fit the grid
   fresh_launch();
-  const dim3 grid((unsigned)(2 * total_blocks)), block(256);
+  const dim3 grid((unsigned)(4 * total_blocks)), block(256);
   hipLaunchKernelGGL(dequantize_batched_kernel, grid, block, 0, (hipStream_t)stream, table, bits,
                      batch_workspace(const_cast<void*>(workspace)), (const uint8_t*)packed_arena,
                      (const uint8_t*)scale_arena, (const uint8_t*)min_arena);
