@@ -1362,23 +1362,25 @@ __host__ __device__ constexpr QGeom q_geom(int bits) {
 // Geometry of the single-tensor dequantize launch for 1, 2, 4 and 8 bit: super-groups per unit, parts a
 // super-group is split into (sgs = 1 then), threads per workgroup, XCD-aware run of tiles - and the same pair
 // (sgs, parts) for large tensors (`large_from` groups and more), with the bytes of dynamic LDS a workgroup
-// of 256 threads asks for there without touching them (0: none; see the occupancy caps below).
+// of 256 threads asks for from `cap_from` groups on without touching them (0: none; see the occupancy caps below).
 // Units are 4 or 8 groups; units of 1 or 2 groups cost 10-150 %: every unit pays its code loads, its table and its
 // divisions.  Dequantize alone, us, units of 4 against units of 8 (no cap), by groups in the tensor:
 //   float 1 bit  65 536: 13.95 / 12.29   100 000: 20.0 / 18.4    (2 and 4 bit alike: 8)
 //   float 8 bit  65 536: 15.76 / 15.98   100 000: 23.2 / 23.7    (4, and 8 with the cap from 2^17 groups)
-//   half  1 bit  16 384: 3.86 / 4.36   65 536: 7.36 / 7.87   100 000: 11.3 / 11.3   130 000: 14.2 / 13.3
+//   half  1 bit  16 384: 3.86 / 4.36   65 536: 6.8 / 7.4   81 920: 10.3 / 8.8   98 304: 10.4 / 10.4   130 000: 14.2 / 13.3
+//                (8 from 73 728 groups; capped at 6 workgroups per CU from 2^18 groups: 67 M elements 25.7 -> 24.8 us, 134 M
+//                48.8 -> 46.7, 268 M 98.3 -> 90.4, while the same cap costs 6-12 % at 29-34 M; 2 and 4 bit lose 2-30 % by any cap)
 //   half  2 bit  16 384: 3.87 / 4.73   65 536: 7.41 / 8.15   130 000: 14.5 / 13.8   1 M: 94.6 / 99.4   (4 throughout)
 //   half  4 bit  16 384: 4.39 / 5.05   65 536: 8.08 / 8.95   200 000: 24.0 / 24.0   401 408: 45.0 / 46.7   1 M: 105.1 / 106.7
 //   half  8 bit  65 536: 9.21 / 9.40   130 000: 18.0 / 18.2
-struct DqGeom { int sgs, parts, threads, run, sgs_large, parts_large; unsigned lds_large; int large_from; };
+struct DqGeom { int sgs, parts, threads, run, sgs_large, parts_large; unsigned lds_large; int large_from, cap_from; };
 #ifndef GACT_DQGEOM_F32
-#define GACT_DQGEOM_F32 {{1, 1, 256, GACT_XCD_RUN_DQ, 1, 1, 53000u, 1 << 17}, {2, 1, 256, GACT_XCD_RUN_DQ, 2, 1, 53000u, 1 << 17}, \
-                         {4, 1, 256, GACT_XCD_RUN_DQ, 4, 1, 53000u, 1 << 17}, {4, 1, 256, GACT_XCD_RUN_DQ, 8, 1, 53000u, 1 << 17}}
+#define GACT_DQGEOM_F32 {{1, 1, 256, GACT_XCD_RUN_DQ, 1, 1, 53000u, 1 << 17, 1 << 17}, {2, 1, 256, GACT_XCD_RUN_DQ, 2, 1, 53000u, 1 << 17, 1 << 17}, \
+                         {4, 1, 256, GACT_XCD_RUN_DQ, 4, 1, 53000u, 1 << 17, 1 << 17}, {4, 1, 256, GACT_XCD_RUN_DQ, 8, 1, 53000u, 1 << 17, 1 << 17}}
 #endif
 #ifndef GACT_DQGEOM_F16
-#define GACT_DQGEOM_F16 {{1, 2, 256, GACT_XCD_RUN_DQ, 1, 1, 0u, 3 << 15}, {1, 1, 256, GACT_XCD_RUN_DQ, 1, 1, 0u, 1 << 17}, \
-                         {2, 1, 256, GACT_XCD_RUN_DQ, 2, 1, 0u, 3 << 15}, {4, 1, 256, GACT_XCD_RUN_DQ, 8, 1, 40000u, 1 << 17}}
+#define GACT_DQGEOM_F16 {{1, 2, 256, GACT_XCD_RUN_DQ, 1, 1, 26000u, 9 << 13, 1 << 18}, {1, 1, 256, GACT_XCD_RUN_DQ, 1, 1, 0u, 1 << 17, 1 << 17}, \
+                         {2, 1, 256, GACT_XCD_RUN_DQ, 2, 1, 0u, 3 << 15, 3 << 15}, {4, 1, 256, GACT_XCD_RUN_DQ, 8, 1, 40000u, 1 << 17, 1 << 17}}
 #endif
 template <typename T>
 __host__ __device__ constexpr DqGeom dq_geom(int bits) {
@@ -2454,7 +2456,7 @@ LaunchPlan plan_dequantize(int bits, int64_t N) {
   const int64_t units_per_block = d.threads / (GROUP / (16 / (int64_t)sizeof(T)));
   const int64_t unit_groups = dq_unit_groups(d, bits, large);
   // the caps are stated for workgroups of 256 threads
-  p.lds = large ? d.lds_large * (unsigned)d.threads / 256u : 0u;
+  p.lds = N >= d.cap_from ? d.lds_large * (unsigned)d.threads / 256u : 0u;
   p.grid = dim3((unsigned)(((N + unit_groups - 1) / unit_groups + units_per_block - 1) / units_per_block));
   p.block = dim3((unsigned)d.threads);
 #define GACT_DQ_KERNEL(B) (large ? (const void*)dequantize_kernel<T, B, true> : (const void*)dequantize_kernel<T, B, false>)

@@ -383,9 +383,11 @@ def test_occupancy_caps_are_what_the_launches_get():
         assert (threads, per_cu) == (256, 3) and lds > 0, (bits, threads, lds, per_cu)
         threads, lds, per_cu = geometry(DQ, _abi.F32, bits, small)
         assert threads == 256 and lds == 0 and per_cu >= 6, (bits, per_cu)
-    # dequantize, half: capped at 8 bit only (4 workgroups)
+    # dequantize, half: capped at 8 bit (4 workgroups) and, from 2^18 groups on, at 1 bit (6 workgroups)
     assert geometry(DQ, _abi.F16, 8, big)[1:] == (40000, 4)
-    for bits in (1, 2, 4):
+    assert geometry(DQ, _abi.F16, 1, big)[1:] == (26000, 6) and geometry(DQ, _abi.BF16, 1, big)[1:] == (26000, 6)
+    assert geometry(DQ, _abi.F16, 1, 1 << 17)[1] == 0 and geometry(DQ, _abi.F16, 1, 1 << 17)[2] >= 7
+    for bits in (2, 4):
         assert geometry(DQ, _abi.F16, bits, big)[1] == 0 and geometry(DQ, _abi.F16, bits, big)[2] >= 6
     # quantize, float: 16 one-wave workgroups per compute unit at 4 bit, 8 at 2 bit, on large tensors only
     assert geometry(Q, _abi.F32, 4, big) == (64, 10000, 16)
