@@ -58,8 +58,8 @@ TRAFFIC_BYTES = {
     ("config3-probs", "dequantize"): 304.15e6,  # 35.71 MB read + 268.44 MB written; algorithmic 304.09 MB
     ("config4", "quantize"): 180.96e6,    # 173.58 MB read + 7.38 MB written; algorithmic 180.18 MB
     ("config4", "dequantize"): 180.34e6,  # 6.84 MB read + 173.50 MB written; algorithmic 180.18 MB
-    ("config5", "quantize"): 4143.22e6,    # 3661.83 MB read + 481.39 MB written; algorithmic 4142.23 MB
-    ("config5", "dequantize"): 4143.55e6,  # 482.71 MB read + 3660.84 MB written; algorithmic 4142.23 MB
+    ("config5", "quantize"): 4143.30e6,    # 3661.91 MB read + 481.39 MB written; algorithmic 4142.23 MB
+    ("config5", "dequantize"): 4144.32e6,  # 483.48 MB read + 3660.84 MB written; algorithmic 4142.23 MB
 }
 
 BASELINE_METRIC = "quantize+dequantize GB/s and % of HBM peak, 1×MI355X, 2-bit group=256"
