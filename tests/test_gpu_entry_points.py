@@ -408,3 +408,29 @@ def test_occupancy_caps_are_what_the_launches_get():
     assert lib.gact_launch_geometry(0, 7, 4, 100, None, None, None) == -1
     assert lib.gact_launch_geometry(1, _abi.F16, 4, 0, None, None, None) == -1
     assert lib.gact_launch_geometry(1, _abi.F16, 4, 100, None, None, None) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+def test_fused_quantize_also_writes_the_maxima_when_asked(dtype, bits):
+    """gact_quantize's optional `mx` output: the per-group maxima of minimax (minimax_cuda_kernel.cu:23-67) from the
+    same pass, for small tensors (at 1 bit: the wave-per-super-group kernel), large ones, and ragged ends."""
+    lib = _abi.lib()
+    torch.manual_seed(3)
+    for numel in (256 * 37 + 100, 256 * 8, 256 * 70001 + 17):
+        x = (torch.randn(numel) * 2).to(dtype)
+        N = (numel + 255) // 256
+        xd = x.cuda()
+        packed = torch.empty((lib.gact_packed_bytes(bits, N, 1, 256) + 1,), dtype=torch.int8, device="cuda")
+        sc, mn, mx = (torch.empty((N,), dtype=dtype, device="cuda") for _ in range(3))
+        _abi.check(lib.gact_quantize(xd.data_ptr(), _abi.dtype_code(dtype), numel, bits, _abi.NOISE_FAST, 5, None,
+                                     packed.data_ptr(), sc.data_ptr(), mn.data_ptr(), mx.data_ptr(),
+                                     torch.cuda.current_stream().cuda_stream))
+        padded = torch.zeros(N * 256, dtype=dtype)
+        padded[:numel] = x
+        rmn, rmx = oracle.minimax(padded.reshape(N, 256).numpy())
+        np.testing.assert_array_equal(mn.cpu().numpy(), rmn)
+        np.testing.assert_array_equal(mx.cpu().numpy(), rmx)
+        ref = oracle.op_quantize(x.numpy(), bits, oracle.NOISE_FAST, 5)
+        np.testing.assert_array_equal(packed.cpu().numpy().view(np.uint8)[:ref[0].size], ref[0])
+        np.testing.assert_array_equal(sc.cpu().numpy(), ref[2].reshape(-1))
