@@ -2273,15 +2273,15 @@ quantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int32_
 // Dequantize, one launch for all widths (every width fits 60 registers): the width of a block's tensor is read
 // from device memory and selects the code path, so no workgroup is launched only to leave.
 template <int BITS>
-__device__ __forceinline__ void dequantize_batched_block(const gact_batch_entry& ent, int64_t lb, int half,
+__device__ __forceinline__ void dequantize_batched_block(const gact_batch_entry& ent, int64_t lb, int quarter,
                                                          const uint8_t* packed, const uint8_t* sc, const uint8_t* mn) {
   const int64_t N = (ent.numel + GROUP - 1) / GROUP;
   if (ent.dtype == GACT_F32)
-    dequantize_block128<float, BITS>(packed, (const float*)sc, (const float*)mn, ent.numel, N, lb, half, (float*)ent.x);
+    dequantize_block128<float, BITS>(packed, (const float*)sc, (const float*)mn, ent.numel, N, lb, quarter, (float*)ent.x);
   else if (ent.dtype == GACT_F16)
-    dequantize_block128<f16, BITS>(packed, (const f16*)sc, (const f16*)mn, ent.numel, N, lb, half, (f16*)ent.x);
+    dequantize_block128<f16, BITS>(packed, (const f16*)sc, (const f16*)mn, ent.numel, N, lb, quarter, (f16*)ent.x);
   else
-    dequantize_block128<bf16, BITS>(packed, (const float*)sc, (const bf16*)mn, ent.numel, N, lb, half, (bf16*)ent.x);
+    dequantize_block128<bf16, BITS>(packed, (const float*)sc, (const bf16*)mn, ent.numel, N, lb, quarter, (bf16*)ent.x);
 }
 // grid: four workgroups per block of 128 groups
 __global__ void __launch_bounds__(256)
@@ -2292,7 +2292,7 @@ dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int3
   // the XCD-aware order of the single-tensor kernel (715 -> 709 us on 120 half tensors)
   const uint32_t tile = xcd_tile<GACT_XCD_RUN_DQB>(blockIdx.x, gridDim.x);
   const int64_t block = tile >> 2;
-  const int half = tile & 3;   // which quarter of the block
+  const int quarter = tile & 3;   // which quarter of the block
   const int t = ws.block_tensor[block];
   const gact_batch_entry ent = table[t];
   const int64_t lb = block - ent.first_block;
@@ -2300,10 +2300,10 @@ dequantize_batched_kernel(const gact_batch_entry* __restrict__ table, const int3
   const uint8_t* sc = scale_arena + ent.stats_offset * 4;
   const uint8_t* mn = min_arena + ent.stats_offset * 4;
   switch (bits[t]) {
-    case 1: dequantize_batched_block<1>(ent, lb, half, packed, sc, mn); break;
-    case 2: dequantize_batched_block<2>(ent, lb, half, packed, sc, mn); break;
-    case 4: dequantize_batched_block<4>(ent, lb, half, packed, sc, mn); break;
-    default: dequantize_batched_block<8>(ent, lb, half, packed, sc, mn); break;
+    case 1: dequantize_batched_block<1>(ent, lb, quarter, packed, sc, mn); break;
+    case 2: dequantize_batched_block<2>(ent, lb, quarter, packed, sc, mn); break;
+    case 4: dequantize_batched_block<4>(ent, lb, quarter, packed, sc, mn); break;
+    default: dequantize_batched_block<8>(ent, lb, quarter, packed, sc, mn); break;
   }
 }
 
