@@ -359,3 +359,50 @@ def test_seed_offset_in_device_memory_equals_the_sum_on_the_host(dtype):
             assert torch.equal(a[0][:-1], b[0][:-1]) and torch.equal(a[2], b[2]) and torch.equal(a[3], b[3])
     with pytest.raises(RuntimeError):
         ops.op_quantize(x, 4, 7, seed_offset=offset.int())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+def test_stochastic_rounding_statistics_of_both_streams_on_the_gpu(dtype, bits):
+    """What the task asks of the stochastic streams: mean error within 1e-3 of the range, and the variance of
+    stochastic rounding, step^2 * f (1 - f), for the library's own stream exactly as for the reference's.  Per element
+    over 2048 seeds' worth of draws (the same group at 2048 positions), and over a 4 M-element tensor."""
+    qmax = 2 ** bits - 1
+    # (a) one group repeated: every position draws its own noise, so a column is 2048 draws for one value
+    torch.manual_seed(21)
+    group = torch.rand(256)
+    group[0], group[1] = 0.0, 1.0
+    x = group.repeat(2048, 1).to(dtype).cuda()
+    xf = x.float()
+    stats = {}
+    for stream in ("reference", "fast"):
+        out = ops.op_dequantize(ops.op_quantize(x, bits, 77, rng_stream=stream), x.shape).float()
+        err = out - xf
+        stats[stream] = (err.mean(dim=0), err.var(dim=0))
+        step = 1.0 / qmax
+        # per value: the mean over 2048 draws within 4 sigma of zero (+ the half-precision grid), overall within 1e-3
+        assert float(err.mean().abs()) < 1e-3, (stream, float(err.mean()))
+        assert float(err.mean(dim=0).abs().max()) < 4 * 0.5 * step / 2048 ** 0.5 + 2e-3
+    if dtype == torch.float32:
+        f = (group.double() * qmax) % 1.0
+        want = ((1.0 / qmax) ** 2 * f * (1 - f)).sum().item()
+        for stream in stats:
+            assert abs(stats[stream][1].double().sum().item() / want - 1) < 0.05, stream
+    # half at 8 bit: the group's maximum can code 2^8, which the reference's uint8 accumulator wraps to 0 (an error of the
+    # whole range, reproduced bit for bit and rare): keep that one column out of the comparison of the variances
+    keep = torch.ones(256, dtype=torch.bool, device="cuda")
+    if dtype == torch.float16 and bits == 8:
+        keep[1] = False
+    ratio = stats["fast"][1][keep].double().sum().item() / stats["reference"][1][keep].double().sum().item()
+    assert abs(ratio - 1) < 0.05, ratio
+    # (b) a whole tensor: mean error and mean squared error of the two streams agree
+    y = torch.rand(16384, 256, generator=torch.Generator().manual_seed(5)).to(dtype).cuda()
+    yf = y.float()
+    mse = {}
+    for stream in ("reference", "fast"):
+        out = ops.op_dequantize(ops.op_quantize(y, bits, 3, rng_stream=stream), y.shape).float()
+        e = out - yf
+        assert float(e.mean().abs()) < 1e-3                      # range is 1
+        # (half at 8 bit: without the rare wrapped maxima, whose count differs between any two streams)
+        mse[stream] = float((e.double() ** 2)[e.abs() < 0.5].mean())
+    assert abs(mse["fast"] / mse["reference"] - 1) < 0.02, mse
