@@ -2789,7 +2789,7 @@ int gact_calc_precision_device(int32_t* b, const float* C, const int64_t* w, int
 }
 
 int64_t gact_batch_workspace_bytes(int64_t L, int64_t total_blocks) {
-  if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x3fffffffLL) return GACT_EINVAL;
+  if (L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x1fffffffLL) return GACT_EINVAL;
   return batch_workspace_need(L, total_blocks);
 }
 
@@ -2827,7 +2827,7 @@ int quantize_batched_on(const gact_batch_entry* table, const int32_t* bits, int6
 }
 
 inline int batched_args_ok(int64_t L, int64_t total_blocks) {
-  return !(L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x3fffffffLL);
+  return !(L < 0 || L > (1 << 30) || total_blocks < 0 || total_blocks > 0x1fffffffLL);   // the dequantize grid is 4 * total_blocks
 }
 }  // namespace
 
@@ -2864,7 +2864,6 @@ int gact_dequantize_batched(const gact_batch_entry* table, const int32_t* bits, 
   if (L == 0 || total_blocks == 0) return GACT_OK;
   if (!table || !bits || !workspace || !packed_arena || !scale_arena || !min_arena) return GACT_EINVAL;
   if (!aligned16(packed_arena) || !aligned16(workspace)) return GACT_EALIGN;
-  if (total_blocks > 0x1fffffffLL) return GACT_EINVAL;   // four workgroups per block must fit the grid
   fresh_launch();
   const dim3 grid((unsigned)(4 * total_blocks)), block(256);
   hipLaunchKernelGGL(dequantize_batched_kernel, grid, block, 0, (hipStream_t)stream, table, bits,

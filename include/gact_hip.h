@@ -128,7 +128,8 @@ typedef struct gact_batch_entry {
 } gact_batch_entry;
 
 /* Bytes of device workspace gact_batch_plan fills for a table of L tensors whose grid has total_blocks
- * blocks (the sum of ceil(N_i/128): a block is 128 groups whatever the width).  16-byte aligned memory. */
+ * blocks (the sum of ceil(N_i/128): a block is 128 groups whatever the width).  16-byte aligned memory.
+ * The batched entry points take L <= 2^30 and total_blocks < 2^29 (GACT_EINVAL beyond). */
 int64_t gact_batch_workspace_bytes(int64_t L, int64_t total_blocks);
 
 /* Plan a batched launch from device-resident bits: fills packed_offset of every table entry (256-byte

@@ -112,6 +112,6 @@ def test_static_workspace_limits():
     lib = _abi.lib()
     # beyond the array: refused before anything is launched (the pointers are never touched)
     assert lib.gact_quantize_batched_static(16, 16, 10, 262145, 1 << 20, 3, 0, 16, 16, 16, None, None) == -6
-    assert lib.gact_quantize_batched_static(16, 16, 10, 1 << 29, 1 << 20, 3, 0, 16, 16, 16, None, None) == -6
+    assert lib.gact_quantize_batched_static(16, 16, 10, (1 << 29) - 1, 1 << 20, 3, 0, 16, 16, 16, None, None) == -6
     assert lib.gact_quantize_batched_static(16, 16, 10, 100, 1 << 20, 3, 0, 16, 16, 16, 4, None) == -2      # verdict not 8-byte aligned
     assert b"limit" in lib.gact_strerror(-6)
