@@ -1416,10 +1416,13 @@ quantize_kernel(const T* __restrict__ x, int64_t numel, int64_t N, uint8_t* __re
 // Quantize at 1 bit with a wave per super-group: row r takes groups 2r and 2r + 1 of the 8 whose codes share bytes, the
 // four rows OR their partial bytes together (two ds_bpermute steps on 4 dwords) and each then stores its quarter of the
 // super-group's 256 bytes.  A wave holds 8 KB (float) or 4 KB (half) where a row per super-group makes it hold 32 or
-// 16 KB: on small tensors, where a kernel is mostly its first and last waves, that is 5-15 % (float 2 M elements
-// 5.3 -> 4.8 us, 8 M 9.5 -> 8.3, 13 M 11.5 -> 10.9; half 2 M 5.1 -> 4.7, 4 M 5.4 -> 4.6); from 16 M elements on the two
-// forms are within 2 % of each other (17 M: 13.0 / 13.6, 43 M: 31.4 / 30.6, 103 M: 67.9 / 68.2 us), at 2 bit (two rows
-// per super-group) there is nothing in it at any size.  Same results as quantize_kernel; not for the reference stream.
+// 16 KB and, with its 175 registers, leaves room for two waves per SIMD: 65 536 float groups are exactly one round of
+// such waves, and the row form's time steps up with every further round (65 536 groups 12.9 us, 69 632: 16.2) where
+// this form grows evenly (13.5, 14.4).  Float, us, row form / this form, by groups: 8 192: 5.3 / 4.8   32 768: 9.5 / 8.3
+// 49 152: 11.3 / 10.8   57 344 .. 65 536: 11.8 .. 12.9 / 12.1 .. 13.5   73 728: 16.8 / 14.9   98 304: 19.7 / 19.4
+// 131 072: 25.2 / 24.2   169 343: 31.4 / 30.7   229 376: 40.9 / 40.4   262 144 and more: equal.  Half: 8 192: 5.1 / 4.7
+// 16 384: 5.4 / 4.6   32 768: 6.7 / 6.6   49 152: 8.2 / 8.3   65 536 and more: 9.2 / 9.9 .. 48.8 / 51.2.  At 2 bit (one
+// group per row) there is nothing in it at any size.  Same results as quantize_kernel; not for the reference stream.
 // ------------------------------------------------------------------------------------------------
 #ifndef GACT_W8_RUN
 #define GACT_W8_RUN 32
@@ -2366,10 +2369,10 @@ inline unsigned quantize_lds_cap(size_t elem_size, int bits, int64_t N) {
 // at 2 bit, deterministic, 5.22 us with a row per super-group against 5.37-5.52 us that way, in workgroups of one or
 // four waves, with or without the XCD-aware tile order; 13 M elements 11.3 against 11.4-11.8 us; 103 M 68.1 / 67.6-68.8.)
 #ifndef GACT_W8_BELOW_F32
-#define GACT_W8_BELOW_F32 57344
+#define GACT_W8_BELOW_F32 (1 << 18)
 #endif
 #ifndef GACT_W8_BELOW_F16
-#define GACT_W8_BELOW_F16 49152
+#define GACT_W8_BELOW_F16 40960
 #endif
 #ifndef GACT_W8_THREADS
 #define GACT_W8_THREADS 256
