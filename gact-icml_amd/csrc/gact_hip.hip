@@ -104,6 +104,19 @@ __device__ __forceinline__ void philox4x32(uint32_t c0, uint32_t c1, uint32_t c2
 __device__ __forceinline__ float curand_uniform_map(uint32_t x) {
   return __builtin_fmaf((float)x, 0x1p-32f, 0x1p-33f);
 }
+// The same with the addend held in a register by the caller (uniform_addend(), once per kernel): left to itself the
+// compiler builds the addend anew in front of every multiply-add, one instruction in nine of a kernel that is bound by
+// its instruction count.
+__device__ __forceinline__ float uniform_addend() {
+  float c;
+  asm volatile("v_mov_b32 %0, 0x2f000000" : "=v"(c));
+  return c;
+}
+__device__ __forceinline__ float curand_uniform_map(uint32_t x, float addend) {
+  float u;
+  asm("v_fmamk_f32 %0, %1, 0x2f800000, %2" : "=v"(u) : "v"((float)x), "v"(addend));
+  return u;
+}
 // 8-bit centred noise of the fast stream from byte B of a Philox word: (2h - 255) / 512 = (h + 0.5) / 256 - 1/2,
 // exact in float (v_cvt_f32_ubyteB and one fma).
 template <int B>
@@ -285,6 +298,13 @@ template <> struct Elem<float> {
     if (CENTRED) return ANY ? rint_clamp0<true>(y) : centred_code_bits_of_any(y);
     return ANY ? rint_clamp0<true>(y - 0.5f) : code_bits_of_any(y);
   }
+  // elements e (even) and e + 1 of chunk k
+  template <bool ANY>
+  __device__ static __forceinline__ void code2(const Store& st, int k, int e, float mn, float s, float ua, float ub,
+                                               uint32_t& ca, uint32_t& cb) {
+    ca = code1<ANY>(st, k, e, mn, s, ua);
+    cb = code1<ANY>(st, k, e + 1, mn, s, ub);
+  }
   // NEG (with CENTRED): the chunk takes the mirrored draws, -u (the negation folds into the fma)
   template <bool CONST_NOISE, bool ANY, bool CENTRED = false, bool NEG = false>
   __device__ static __forceinline__ void codes(const Store& st, int k, float mn, float s, const float (&u)[4],
@@ -429,6 +449,16 @@ template <> struct Elem<f16> {
     if (CENTRED) return ANY ? centred_code_bits_of_any(y) : centred_code_bits_of(y);
     return ANY ? code_bits_of_any(y) : code_bits_of(y);
   }
+  // elements e (even) and e + 1 of chunk k, one pair: packed subtraction and product, the sum with the widening folded in
+  template <bool ANY>
+  __device__ static __forceinline__ void code2(const Store& st, int k, int e, f16 mn, f16 s, float ua, float ub,
+                                               uint32_t& ca, uint32_t& cb) {
+    const f16x2 mn2 = {mn, mn}, s2 = {s, s};
+    const f16x2 p = (st.v[k][e >> 1] - mn2) * s2;
+    const float ya = widen_add_lo(p, ua), yb = widen_add_hi(p, ub);
+    ca = ANY ? code_bits_of_any(ya) : code_bits_of(ya);
+    cb = ANY ? code_bits_of_any(yb) : code_bits_of(yb);
+  }
   template <bool CONST_NOISE, bool ANY, bool CENTRED = false, bool NEG = false>
   __device__ static __forceinline__ void codes(const Store& st, int k, f16 mn, f16 s, const float (&u)[8],
                                                uint32_t (&c)[8]) {
@@ -549,6 +579,12 @@ template <> struct Elem<bf16> {
     float y = __builtin_fmaf(t, s, u);
     if (CENTRED) return ANY ? rint_clamp0<true>(y) : centred_code_bits_of(y);
     return ANY ? rint_clamp0<true>(y - 0.5f) : code_bits_of(y);
+  }
+  template <bool ANY>
+  __device__ static __forceinline__ void code2(const Store& st, int k, int e, float mn, float s, float ua, float ub,
+                                               uint32_t& ca, uint32_t& cb) {
+    ca = code1<ANY>(st, k, e, mn, s, ua);
+    cb = code1<ANY>(st, k, e + 1, mn, s, ub);
   }
   template <bool CONST_NOISE, bool ANY, bool CENTRED = false, bool NEG = false>
   __device__ static __forceinline__ void codes(const Store& st, int k, float mn, float s, const float (&u)[8],
@@ -904,20 +940,28 @@ __device__ __forceinline__ void quantize_supergroup(const T* __restrict__ x, int
       for (int e = 0; e < W; e++) bytes[k][e] = 0;
 
     if (NOISE == GACT_NOISE_REF) {
-      // one Philox state per output byte j: key = seed, counter = (draw/4, 0, j lo, j hi)
+      // one Philox state per output byte j: key = seed, counter = (draw/4, 0, j lo, j hi); two neighbouring bytes at
+      // a time, so that the half path can take its elements in pairs
+      const float addend = uniform_addend();
 #pragma unroll
       for (int k = 0; k < CH; k++)
 #pragma unroll
-        for (int e = 0; e < W; e++) {
+        for (int e = 0; e < W; e += 2) {
           const uint64_t j = (uint64_t)sg * GROUP + chunk_col<T>(k, i) + e;
-          uint32_t r[4];
+          uint32_t ra[4], rb[4];
 #pragma unroll
           for (int ni = 0; ni < WPT; ni++) {
             const int g = q * WPT + ni;
-            if ((ni & 3) == 0) philox4x32<PHILOX_REF_ROUNDS>(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, r);
+            if ((ni & 3) == 0) {
+              philox4x32<PHILOX_REF_ROUNDS>(ni >> 2, 0u, (uint32_t)j, (uint32_t)(j >> 32), k0, k1, ra);
+              philox4x32<PHILOX_REF_ROUNDS>(ni >> 2, 0u, (uint32_t)(j + 1), (uint32_t)((j + 1) >> 32), k0, k1, rb);
+            }
             if (n0 + g < N) {
-              float u = curand_uniform_map(r[ni & 3]);
-              bytes[k][e] |= Elem<T>::template code1<GIVEN>(v[g], k, e, lo_t[g], s_t[g], u) << (ni * BITS);
+              uint32_t ca, cb;
+              Elem<T>::template code2<GIVEN>(v[g], k, e, lo_t[g], s_t[g], curand_uniform_map(ra[ni & 3], addend),
+                                             curand_uniform_map(rb[ni & 3], addend), ca, cb);
+              bytes[k][e] |= ca << (ni * BITS);
+              bytes[k][e + 1] |= cb << (ni * BITS);
             }
           }
         }
