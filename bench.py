@@ -25,7 +25,8 @@ Beside the workloads the line carries what plain streams reach in the same run: 
 pure read, torch's element-wise kernel at the 8:1 and 1:8 read:write mixes, and the duration of a one-group
 launch, on config2's tensor), `ceilings_headline` (the same on config1's tensor) and `ceilings_by_size` (fill and
 pure read at the sizes of the mid-sized workloads); `configs["config1-cached"]` is the headline tensor with one
-buffer set.
+buffer set.  `entry_points` times the entry points no workload goes through (gact_pack with the caller's min / max,
+gact_unpack, the dropout-mask bit packing) on config2's tensor.
 
 Prints ONE JSON line.
 """
@@ -336,6 +337,73 @@ def run_ceilings(torch, timer, name="config2", full=True):
     return out
 
 
+def run_entry_points(torch, timer, name="config2", seed=42):
+    """The entry points no workload above goes through, each alone on config2's tensor: the reference's
+    three-step quantize (gact_minimax, then gact_pack with the caller's min / max; gact_unpack is the way back)
+    and the dropout-mask bit packing on a mask with one byte per element of that tensor."""
+    from gact.cpp_extension import _abi
+
+    lib = _abi.lib()
+    shape, dtype, bits, stream, kind, _ = WORKLOADS[name]
+    x0 = make_input(torch, shape, dtype, kind)
+    n = x0.numel()
+    N = n // 256
+    esize = x0.element_size()
+    packed_len = lib.gact_packed_bytes(bits, N, 1, 256)
+    sets = max(1, -(-ROTATE_BYTES // (n * esize + packed_len)))
+    xs = [x0 if r == 0 else x0.clone() for r in range(sets)]
+    ys = [torch.empty_like(x0) for _ in range(sets)]
+    qs = [torch.empty((packed_len,), dtype=torch.int8, device="cuda") for _ in range(sets)]
+    mn, mx, sc = (torch.empty((N,), dtype=x0.dtype, device="cuda") for _ in range(3))
+    mode = {"deterministic": _abi.NOISE_CONST, "reference": _abi.NOISE_REF, "fast": _abi.NOISE_FAST}[stream]
+    code = _abi.dtype_code(x0.dtype)
+
+    def st():
+        return torch.cuda.current_stream().cuda_stream
+
+    _abi.check(lib.gact_minimax(x0.data_ptr(), code, N, 256, mn.data_ptr(), mx.data_ptr(), st()))
+
+    def pack(k):
+        _abi.check(lib.gact_pack(xs[k % sets].data_ptr(), mn.data_ptr(), mx.data_ptr(), code, bits, N, 1, 256, mode, seed + k,
+                                 None, qs[k % sets].data_ptr(), sc.data_ptr(), st()))
+
+    def unpack(k):
+        _abi.check(lib.gact_unpack(qs[k % sets].data_ptr(), bits, sc.data_ptr(), mn.data_ptr(), code, N, 1, 256,
+                                   ys[k % sets].data_ptr(), st()))
+
+    for k in range(sets):
+        pack(k)
+    out = {"tensor": "%s's (%d bytes), %d bit" % (name, n * esize, bits), "buffer_sets": sets}
+    for key, fn, moved in (("pack", pack, n * esize + packed_len + 3 * esize * N),
+                           ("unpack", unpack, n * esize + packed_len + 2 * esize * N)):
+        ms, _ = timer(fn, sets)
+        out[key] = {"us": ms * 1e3, "gbs": moved / (ms * 1e-3) / 1e9, "frac": moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    del xs, ys, qs
+    torch.cuda.empty_cache()
+    words = (n + 31) // 32
+    msets = max(1, -(-ROTATE_BYTES // (n + 4 * words)))
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    m0 = (torch.rand((n,), device="cuda", generator=g) < 0.9).to(torch.uint8)
+    ms_ = [m0 if r == 0 else m0.clone() for r in range(msets)]
+    ws = [torch.empty((words,), dtype=torch.int32, device="cuda") for _ in range(msets)]
+
+    def mask_pack(k):
+        _abi.check(lib.gact_mask_pack(ms_[k % msets].data_ptr(), n, ws[k % msets].data_ptr(), st()))
+
+    def mask_unpack(k):
+        _abi.check(lib.gact_mask_unpack(ws[k % msets].data_ptr(), n, ms_[k % msets].data_ptr(), st()))
+
+    for k in range(msets):
+        mask_pack(k)
+    for key, fn in (("mask_pack", mask_pack), ("mask_unpack", mask_unpack)):
+        ms, _ = timer(fn, msets)
+        moved = n + 4 * words
+        out[key] = {"us": ms * 1e3, "gbs": moved / (ms * 1e-3) / 1e9, "frac": moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                    "bytes": moved}
+    return out
+
+
 def run_config5(torch, timer, seed=42):
     """Workload "config5", the full adaptive step: 120 fp16 tensors with Swin-Tiny-like shapes, per-tensor
     sensitivities ~LogNormal(0,2), budget 2 bits per element.  One step = greedy calc_precision on the GPU
@@ -579,6 +647,8 @@ def main():
         configs["reference-test-speed"]["python_ops_us"] = python_ops_us(torch, "reference-test-speed", args.min_seconds)
         line["configs"] = configs
         line["ceilings"] = run_ceilings(torch, timer, "config2")
+        torch.cuda.empty_cache()
+        line["entry_points"] = run_entry_points(torch, timer, "config2")
         torch.cuda.empty_cache()
         # the same plain streams at the headline workload's size, where the launch and the ramp of a 16 MB
         # stream count: what a kernel that only reads (or only fills) this tensor takes

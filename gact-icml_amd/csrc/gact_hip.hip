@@ -1815,7 +1815,9 @@ unpack_rows8_kernel(const uint8_t* __restrict__ packed, int bits, const T* __res
 // e/32, bit e%32), which is the plain ballot of one byte per lane and fits the ceil(n/32)-word output.
 // ------------------------------------------------------------------------------------------------
 // A wave takes MASK_PAIRS consecutive pairs of blocks (4 KB of mask bytes) and issues all its loads first.
+#ifndef MASK_PAIRS
 #define MASK_PAIRS 4
+#endif
 __global__ void __launch_bounds__(256)
 mask_pack_kernel(const uint8_t* __restrict__ data, int64_t n, int32_t* __restrict__ mask) {
   const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
