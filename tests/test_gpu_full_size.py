@@ -132,14 +132,15 @@ def test_config3_bert_large_fp16(name, shape, kind, bits):
     cross_check_kernel_paths(x, q, bits, "fast", 7)
 
 
-@pytest.mark.parametrize("groups", [32768 + 3, 100000 + 3, 196608 + 3])
+@pytest.mark.parametrize("groups", [32768 + 3, 100000 + 3, 196608 + 3, 262144 + 3])
 @pytest.mark.parametrize("bits", [1, 2, 4, 8])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_large_tensor_launches(dtype, bits, groups):
-    """Large tensors take their own dequantize geometry (from 98 304 or 131 072 groups on) and some kernels are
+    """Large tensors take their own dequantize geometry (from 73 728, 98 304 or 131 072 groups on) and some kernels are
     launched with fewer resident waves per CU (a request for dynamic LDS that they never touch; the last of those
-    sizes is 196 608 groups), and quantize changes how its rows are worked through at 32 768 groups: every type and
-    width just past the first, the middle and the last of those sizes, with a partial last super-group."""
+    sizes is 262 144 groups), quantize changes how its rows are worked through at 32 768 groups, and 1 bit leaves the
+    wave-per-super-group kernel at 40 960 (half) and 262 144 groups (float): every type and width just past the first,
+    the middle and the last of those sizes, with a partial last super-group."""
     x = gen((groups, 256), dtype, "relu", 5)
     q, out = check_against_oracle(x, bits, "fast", 13)
     check_properties(x, q, out, bits, stochastic=True)
