@@ -47,20 +47,24 @@ MIN_SECONDS = 1.0      # every timed loop runs at least this long
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size
 # in the same runs (profiles/<workload>_*.txt name the runs and the factors); absent = no counter run
 TRAFFIC_BYTES = {
-    ("config1", "quantize"): 18.07e6,    # 16.85 MB read + 1.22 MB written; algorithmic 17.96 MB
+    ("config1", "quantize"): 18.06e6,    # 16.84 MB read + 1.22 MB written; algorithmic 17.96 MB
     ("config1", "dequantize"): 18.02e6,  # 1.25 MB read + 16.78 MB written; algorithmic 17.96 MB
-    ("config2", "quantize"): 468.31e6,    # 411.06 MB read + 57.24 MB written; algorithmic 465.63 MB
-    ("config2", "dequantize"): 465.69e6,  # 54.65 MB read + 411.04 MB written; algorithmic 465.63 MB
+    ("config2", "quantize"): 468.27e6,    # 411.06 MB read + 57.21 MB written; algorithmic 465.63 MB
+    ("config2", "dequantize"): 465.68e6,  # 54.64 MB read + 411.04 MB written; algorithmic 465.63 MB
     ("config3-hidden", "quantize"): 50.63e6,    # 33.59 MB read + 17.04 MB written; algorithmic 50.59 MB
-    ("config3-hidden", "dequantize"): 50.69e6,  # 17.14 MB read + 33.55 MB written; algorithmic 50.59 MB
-    ("config3-gelu", "quantize"): 168.88e6,    # 134.27 MB read + 34.60 MB written; algorithmic 168.82 MB
+    ("config3-hidden", "dequantize"): 50.69e6,  # 17.13 MB read + 33.55 MB written; algorithmic 50.59 MB
+    ("config3-gelu", "quantize"): 168.87e6,    # 134.27 MB read + 34.60 MB written; algorithmic 168.82 MB
     ("config3-gelu", "dequantize"): 168.88e6,  # 34.66 MB read + 134.22 MB written; algorithmic 168.82 MB
     ("config3-probs", "quantize"): 304.20e6,    # 268.55 MB read + 35.65 MB written; algorithmic 304.09 MB
     ("config3-probs", "dequantize"): 304.15e6,  # 35.71 MB read + 268.44 MB written; algorithmic 304.09 MB
+    ("config2-refstream", "quantize"): 467.41e6,    # 411.15 MB read + 56.26 MB written; algorithmic 465.63 MB
+    ("config2-refstream", "dequantize"): 465.68e6,  # 54.64 MB read + 411.04 MB written; algorithmic 465.63 MB
+    ("config3-probs-refstream", "quantize"): 304.29e6,    # 268.64 MB read + 35.65 MB written; algorithmic 304.09 MB
+    ("config3-probs-refstream", "dequantize"): 304.15e6,  # 35.71 MB read + 268.44 MB written; algorithmic 304.09 MB
     ("config4", "quantize"): 180.23e6,    # 173.46 MB read + 6.77 MB written; algorithmic 180.18 MB
-    ("config4", "dequantize"): 180.34e6,  # 6.84 MB read + 173.50 MB written; algorithmic 180.18 MB
-    ("config5", "quantize"): 4143.30e6,    # 3661.91 MB read + 481.39 MB written; algorithmic 4142.23 MB
-    ("config5", "dequantize"): 4144.32e6,  # 483.48 MB read + 3660.84 MB written; algorithmic 4142.23 MB
+    ("config4", "dequantize"): 180.33e6,  # 6.84 MB read + 173.49 MB written; algorithmic 180.18 MB
+    ("config5", "quantize"): 4143.29e6,    # 3661.90 MB read + 481.39 MB written; algorithmic 4142.23 MB
+    ("config5", "dequantize"): 4144.33e6,  # 483.49 MB read + 3660.84 MB written; algorithmic 4142.23 MB
 }
 
 BASELINE_METRIC = "quantize+dequantize GB/s and % of HBM peak, 1×MI355X, 2-bit group=256"
